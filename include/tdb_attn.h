@@ -154,13 +154,6 @@ int tdb_delta_table(int32_t* out, int32_t max_len, int32_t position_buckets, int
  */
 int tdb_check_cu_seqlens(const int32_t* cu_seqlens_host, int32_t batch, int32_t total_tokens, int32_t max_seqlen);
 
-/*
- * Host-only.  Number of workgroups tdb_attn_fwd_varlen launches along x for the given sizes and
- * the query-tile height it will pick; an upper bound sum_b ceil(len_b / tile) <=
- * total_tokens / tile + batch that needs no knowledge of the lengths.
- */
-int tdb_varlen_grid(int32_t dtype, int32_t head_dim, int32_t total_tokens, int32_t batch, int32_t* tile_rows);
-
 #ifdef __cplusplus
 }
 #endif

@@ -141,8 +141,6 @@ def test_varlen_argument_validation():
     assert _lib.ERROR_NAMES[lib.tdb_attn_fwd_varlen(C.byref(a), None)] == "TDB_ERR_SHAPE"
     a.total_tokens = 0
     assert lib.tdb_attn_fwd_varlen(C.byref(a), None) == 0
-    tile = C.c_int32()
-    assert lib.tdb_varlen_grid(_lib.TDB_F32, 64, 1000, 10, C.byref(tile)) == 1000 // tile.value + 10
 
 
 def test_operators_refuse_cpu_tensors():

@@ -16,6 +16,7 @@ SOURCES = ("capi.hip", "attn_generic.hip", "attn_mfma.hip")
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-mllvm", "-amdgpu-mfma-vgpr-form=1",      # MFMA accumulators in VGPRs: no accvgpr copies around the softmax
     "-Wno-unused-command-line-argument",
     "-I", os.path.join(ROOT, "include"), "-I", CSRC,
 ]

@@ -26,7 +26,7 @@ ERROR_NAMES = {
 _VALUE_ERRORS = {-1, -2, -3, -4, -5, -6, -7, -8, -9}
 
 EXPORTS = ("tdb_version", "tdb_last_error", "tdb_attn_fwd_fixed", "tdb_attn_fwd_varlen", "tdb_bucket_table",
-           "tdb_delta_table", "tdb_check_cu_seqlens", "tdb_varlen_grid")
+           "tdb_delta_table", "tdb_check_cu_seqlens")
 
 
 class PosArgs(C.Structure):
@@ -99,8 +99,6 @@ def load() -> C.CDLL:
             fn.restype = C.c_int
         lib.tdb_check_cu_seqlens.argtypes = [C.c_void_p, C.c_int32, C.c_int32, C.c_int32]
         lib.tdb_check_cu_seqlens.restype = C.c_int
-        lib.tdb_varlen_grid.argtypes = [C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.POINTER(C.c_int32)]
-        lib.tdb_varlen_grid.restype = C.c_int
         if lib.tdb_version() != ABI_VERSION:
             raise RuntimeError(f"libtdb_attn.so has ABI {lib.tdb_version()}, this package expects {ABI_VERSION}")
         _lib = lib

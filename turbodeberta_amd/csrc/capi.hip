@@ -166,13 +166,6 @@ int tdb_check_cu_seqlens(const int32_t* cu, int32_t batch, int32_t total_tokens,
     return TDB_OK;
 }
 
-int tdb_varlen_grid(int32_t dtype, int32_t head_dim, int32_t total_tokens, int32_t batch, int32_t* tile_rows) {
-    const int tile = (dtype == TDB_BF16 && head_dim == 64) ? TDB_MFMA_TILE : TDB_GENERIC_TILE;
-    if (tile_rows) *tile_rows = tile;
-    if (total_tokens < 0 || batch < 0) return fail(TDB_ERR_SHAPE, "negative size");
-    return total_tokens / tile + batch;
-}
-
 int tdb_attn_fwd_fixed(const tdb_fixed_args* a, void* stream) {
     if (!a) return fail(TDB_ERR_NULL, "args is NULL");
     int rc = check_common(a->dtype, a->batch, a->heads, a->head_dim, a->seqlen, a->causal, a->q, a->k, a->v, a->o);
