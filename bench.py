@@ -1,0 +1,202 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused disentangled-attention forward on one MI355X.
+
+A "step" is one attention forward over one batch of synthetic DeBERTa-v3-base attention inputs
+(12 heads x 64, rel-pos buckets 256 / max 512), bf16, inputs resident in HBM:
+
+  fixed   batch 32 x seq 512, right-padded, valid lengths uniform in [384, 512]   (headline `value`)
+  varlen  64 sequences with lengths uniform in [16, 512], packed with cu_seqlens  (reported beside it)
+
+Prints ONE JSON line.  `value` is algorithmic attention TFLOP/s of the fixed workload over the timed
+region; FLOPs per sequence of valid length l and per head:  4*l*l*d (QK^T + PV) + 4*l*W*d (c2p + p2c),
+W = min(2*span, 2*l - 1) -- no credit for padding, window recompute or projections.
+`roofline` prices the kernel's average launch duration (HIP events on the launch stream) against the
+MI355X dense bf16 MFMA peak; `cpu_baseline` times the CPU oracle (eager float32 restatement of
+Hugging Face's DisentangledSelfAttention) on a bounded sample of the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+H, D, HID = 12, 64, 768
+BUCKETS, MAX_REL, SPAN = 256, 512, 256
+PEAK_BF16_TFLOPS = 2500.0       # MI355X dense bf16 MFMA, AMD public spec
+PEAK_HBM_GBS = 8000.0
+METRIC = "attn TFLOP/s + tokens/s, DeBERTa-v3-base b32xL512 bf16, fixed and varlen"
+
+
+def flops_of(lengths) -> float:
+    tot = 0.0
+    for l in lengths:
+        l = int(l)
+        w = min(2 * SPAN, 2 * l - 1)
+        tot += 4.0 * l * l * D + 4.0 * l * w * D
+    return H * tot
+
+
+def algorithmic_bytes(lengths) -> float:
+    t = float(sum(int(x) for x in lengths))
+    return 2.0 * 4 * t * H * D + 2 * H * 2 * SPAN * D * 2.0
+
+
+def make_weights(dev, seed=0):
+    g = torch.Generator(device=dev).manual_seed(seed)
+    mk = lambda *s, std: (torch.randn(*s, generator=g, device=dev, dtype=torch.float32) * std)
+    w = {n: mk(HID, HID, std=0.02).to(torch.bfloat16) for n in ("wq", "wk", "wv")}
+    w["rel"] = mk(2 * SPAN, HID, std=1.0).to(torch.bfloat16)
+    return w, g
+
+
+def position_tables(w):
+    lin = torch.nn.functional.linear
+    pk = lin(w["rel"], w["wk"]).view(2 * SPAN, H, D).permute(1, 0, 2).contiguous()     # K_r [H, 2s, D]
+    pq = lin(w["rel"], w["wq"]).view(2 * SPAN, H, D).permute(1, 0, 2).contiguous()     # Q_r
+    return pk, pq
+
+
+def build_fixed(dev, B=32, L=512):
+    from turbodeberta_amd.ops import flash_attention as fa
+    w, g = make_weights(dev)
+    lengths = np.random.RandomState(0).randint(384, 513, size=B)
+    hidden = torch.randn(B, L, HID, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    lin = torch.nn.functional.linear
+    heads = lambda x: x.view(B, L, H, D).permute(0, 2, 1, 3)       # projection-native storage, [B,H,L,D] view
+    q, k, v = heads(lin(hidden, w["wq"])), heads(lin(hidden, w["wk"])), heads(lin(hidden, w["wv"]))
+    pk, pq = position_tables(w)
+    lens = torch.from_numpy(lengths.astype(np.int32)).to(dev)
+    plan = fa.prepare(q, k, v, None, None, False, 1.0 / math.sqrt(3 * D), BUCKETS, MAX_REL,
+                      pos_key_layer=pk, pos_query_layer=pq, seqlens_k=lens)
+    return plan, lengths, dict(q=q, k=k, v=v, pk=pk, pq=pq)
+
+
+def build_varlen(dev, n_seq=64):
+    from turbodeberta_amd.ops import flash_attention_varlen as fv
+    w, g = make_weights(dev)
+    lengths = np.random.RandomState(0).randint(16, 513, size=n_seq)
+    T = int(lengths.sum())
+    hidden = torch.randn(T, HID, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    lin = torch.nn.functional.linear
+    q, k, v = (lin(hidden, w[n]).view(T, H, D) for n in ("wq", "wk", "wv"))
+    pk, pq = position_tables(w)
+    cu = torch.from_numpy(np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)).to(dev)
+    plan = fv.prepare(q, k, v, None, None, cu, cu, int(lengths.max()), int(lengths.max()), False,
+                      1.0 / math.sqrt(3 * D), BUCKETS, MAX_REL, pos_key_layer=pk, pos_query_layer=pq)
+    return plan, lengths
+
+
+def time_steps(plan, steps, warmup):
+    """(wall ms per step over exactly `steps` back-to-back launches, mean kernel ms from HIP events)."""
+    for _ in range(warmup):
+        plan.launch()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        plan.launch()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    # per-launch duration: an event pair around every launch on the launch stream
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    for a, b in ev:
+        a.record()
+        plan.launch()
+        b.record()
+    torch.cuda.synchronize()
+    durs = sorted(a.elapsed_time(b) for a, b in ev)
+    return wall_ms, float(np.mean(durs)), durs[len(durs) // 2], durs[0]
+
+
+def cpu_baseline(tensors, lengths, budget_s=12.0):
+    """Oracle (float32 eager restatement of HF) on the first 2 sequences of the fixed workload."""
+    from oracle import hf_eager as O
+    nb = 2
+    f = lambda t: t[:nb].float().cpu().contiguous()
+    q, k, v = f(tensors["q"]), f(tensors["k"]), f(tensors["v"])
+    pk, pq = tensors["pk"].float().cpu(), tensors["pq"].float().cpu()
+    lens = torch.from_numpy(lengths[:nb].astype(np.int32))
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    run = lambda: O.attention_lengths(q, k, v, pk, pq, lens, position_buckets=BUCKETS, max_relative_positions=MAX_REL)
+    run()
+    times, t_start = [], time.perf_counter()
+    while len(times) < 5 or (time.perf_counter() - t_start < budget_s and len(times) < 200):
+        t0 = time.perf_counter()
+        run()
+        times.append(time.perf_counter() - t0)
+    med = float(np.median(times))
+    return {"value": round(flops_of(lengths[:nb]) / med / 1e12, 5), "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+            "kind": "port", "ms_per_sample": round(med * 1e3, 2),
+            "sample": f"first {nb} of the 32 sequences of the fixed workload (lengths {lengths[:nb].tolist()}), "
+                      f"float32 torch-CPU oracle, median of {len(times)} runs"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--workload", choices=["both", "fixed", "varlen"], default="both")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: every figure of this path is per GPU (no collectives); run with --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU: the operators have no CPU implementation", file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device("cuda", int(os.environ.get("LOCAL_RANK", "0")))
+    torch.cuda.set_device(dev)
+
+    out = {"metric": METRIC, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+           "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic"}
+
+    def measure(plan, lengths, name, kernel):
+        wall_ms, mean_ms, med_ms, min_ms = time_steps(plan, args.steps, args.warmup)
+        fl = flops_of(lengths)
+        ach = fl / (mean_ms * 1e-3) / 1e12
+        return {
+            "value": round(fl / (wall_ms * 1e-3) / 1e12, 2), "ms_per_step": round(wall_ms, 4),
+            "tokens_per_s": round(float(lengths.sum()) / (wall_ms * 1e-3), 1),
+            "core_tflops": round(H * sum(4.0 * int(l) ** 2 * D for l in lengths) / (wall_ms * 1e-3) / 1e12, 2),
+            "roofline": {"bound": "mfma", "achieved": round(ach, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                         "frac": round(ach / PEAK_BF16_TFLOPS, 4), "traffic": None, "kernel": kernel,
+                         "kernel_ms_mean": round(mean_ms, 4), "kernel_ms_median": round(med_ms, 4),
+                         "kernel_ms_min": round(min_ms, 4), "algorithmic_gflop": round(fl / 1e9, 3),
+                         "hbm_gbs_algorithmic": round(algorithmic_bytes(lengths) / (mean_ms * 1e-3) / 1e9, 1)},
+        }
+
+    res_fixed = res_var = None
+    tensors = lengths_f = None
+    if args.workload in ("both", "fixed"):
+        plan, lengths_f, tensors = build_fixed(dev)
+        res_fixed = measure(plan, lengths_f, "fixed", "attn_mfma_kernel<c2p,p2c>")
+    if args.workload in ("both", "varlen"):
+        plan_v, lengths_v = build_varlen(dev)
+        res_var = measure(plan_v, lengths_v, "varlen", "attn_mfma_kernel<c2p,p2c>")
+    head = res_fixed or res_var
+    out.update({"value": head["value"], "ms_per_step": head["ms_per_step"], "tokens_per_s": head["tokens_per_s"],
+                "core_tflops": head["core_tflops"], "roofline": head["roofline"]})
+    out["config"] = {"workload": ("fixed b32xL512, valid lengths U[384,512] seed 0" if res_fixed else
+                                  "varlen 64 seqs U[16,512] seed 0") + ", 12 heads x 64, buckets 256, max_rel 512, c2p|p2c",
+                     "global_batch": 32 if res_fixed else 64, "seq_len": 512}
+    if res_fixed and res_var:
+        out["varlen"] = {"workload": "64 packed sequences, lengths U[16,512] seed 0, total tokens %d" % int(lengths_v.sum()),
+                         **res_var}
+    if not args.no_cpu_baseline and tensors is not None:
+        out["cpu_baseline"] = cpu_baseline(tensors, lengths_f)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

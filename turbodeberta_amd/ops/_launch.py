@@ -122,8 +122,24 @@ def default_scale(sm_scale, head_dim: int) -> float:
     return 1.0 / math.sqrt(head_dim) if sm_scale is None else float(sm_scale)
 
 
-def stream_of(dev: torch.device) -> int:
-    return torch.cuda.current_stream(dev).cuda_stream
+class PreparedLaunch:
+    """A fully validated call: the packed argument block, the output tensor and every tensor the
+    block points into.  ``launch()`` issues the kernel on the current stream of the tensors' device
+    and can be repeated (same inputs, same output buffer) at the cost of one C call."""
+
+    __slots__ = ("_fn", "args", "out", "_keep", "_dev")
+
+    def __init__(self, fn, args, out, keep, dev):
+        self._fn, self.args, self.out, self._keep, self._dev = fn, args, out, keep, dev
+
+    def launch(self) -> torch.Tensor:
+        if torch.cuda.current_device() != self._dev.index:      # HIP launches on the current device
+            with torch.cuda.device(self._dev):
+                return self.launch()
+        rc = self._fn(C.byref(self.args), torch.cuda.current_stream(self._dev).cuda_stream)
+        if rc:
+            _lib.check(rc)
+        return self.out
 
 
 BACKWARD_MESSAGE = "Backward pass is not implemented for FlashAttentionDisentangled"

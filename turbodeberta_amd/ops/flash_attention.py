@@ -14,8 +14,9 @@ from .. import _lib
 from . import _launch as L
 
 
-def _forward(q, k, v, q_pos, k_pos, causal, sm_scale, position_buckets, max_relative_distance,
-             pos_key_layer, pos_query_layer, seqlens_k, force_generic):
+def prepare(q, k, v, q_pos, k_pos, causal=False, sm_scale=None, position_buckets=0, max_relative_distance=0, *,
+            pos_key_layer=None, pos_query_layer=None, seqlens_k=None, force_generic=False) -> L.PreparedLaunch:
+    """Validate and pack one call of ``flash_attention_with_disentangled`` without launching it."""
     if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
         raise ValueError("q, k, v must be [B, H, L, D]")
     Dq, Dk, Dv = q.shape[-1], k.shape[-1], v.shape[-1]
@@ -39,7 +40,7 @@ def _forward(q, k, v, q_pos, k_pos, causal, sm_scale, position_buckets, max_rela
     o = torch.empty_like(q)
     if not L.rows_ok(o):
         o = torch.empty(q.shape, dtype=q.dtype, device=dev)
-    keep = []
+    keep = [q, k, v]
 
     a = _lib.FixedArgs()
     a.dtype = L.dtype_code(q)
@@ -74,9 +75,8 @@ def _forward(q, k, v, q_pos, k_pos, causal, sm_scale, position_buckets, max_rela
     L.fill_pos(a.pos, dev=dev, max_len=M, span=span, position_buckets=position_buckets,
                max_relative_distance=max_relative_distance, pos_key=pk, pos_query=pq,
                c2p_strip=strips[0], p2c_strip=strips[1], varlen=False, keep=keep)
-    with torch.cuda.device(dev):
-        _lib.check(_lib.load().tdb_attn_fwd_fixed(C.byref(a), L.stream_of(dev)))
-    return o
+    keep += [t for t in (strips[0], strips[1], pk, pq) if t is not None]
+    return L.PreparedLaunch(_lib.load().tdb_attn_fwd_fixed, a, o, keep, dev)
 
 
 class FlashAttentionDisentangled(torch.autograd.Function):
@@ -85,8 +85,9 @@ class FlashAttentionDisentangled(torch.autograd.Function):
     @staticmethod
     def forward(ctx, q, k, v, q_pos, k_pos, causal, sm_scale, position_buckets, max_relative_distance,
                 pos_key_layer, pos_query_layer, seqlens_k, force_generic):
-        return _forward(q, k, v, q_pos, k_pos, causal, sm_scale, position_buckets, max_relative_distance,
-                        pos_key_layer, pos_query_layer, seqlens_k, force_generic)
+        return prepare(q, k, v, q_pos, k_pos, causal, sm_scale, position_buckets, max_relative_distance,
+                       pos_key_layer=pos_key_layer, pos_query_layer=pos_query_layer, seqlens_k=seqlens_k,
+                       force_generic=force_generic).launch()
 
     @staticmethod
     def backward(ctx, grad_output):

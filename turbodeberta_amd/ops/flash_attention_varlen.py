@@ -16,8 +16,10 @@ from .. import _lib
 from . import _launch as L
 
 
-def _forward(q, k, v, q_pos, k_pos, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, causal, sm_scale,
-             position_buckets, max_relative_distance, pos_key_layer, pos_query_layer, force_generic):
+def prepare(q, k, v, q_pos, k_pos, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, causal=False, sm_scale=None,
+            position_buckets=0, max_relative_distance=0, *, pos_key_layer=None, pos_query_layer=None,
+            force_generic=False) -> L.PreparedLaunch:
+    """Validate and pack one call of ``flash_attention_with_disentangled_varlen`` without launching it."""
     if q.dim() != 3 or k.dim() != 3 or v.dim() != 3:
         raise ValueError("q, k, v must be [total_tokens, H, D]")
     Dq, Dk, Dv = q.shape[-1], k.shape[-1], v.shape[-1]
@@ -46,7 +48,7 @@ def _forward(q, k, v, q_pos, k_pos, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, ma
     if not L.rows_ok(o):
         o = torch.empty(q.shape, dtype=q.dtype, device=dev)
     cu = cu_seqlens_q.to(torch.int32).contiguous()
-    keep = [cu]
+    keep = [cu, q, k, v]
 
     a = _lib.VarlenArgs()
     a.dtype = L.dtype_code(q)
@@ -76,9 +78,8 @@ def _forward(q, k, v, q_pos, k_pos, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, ma
     L.fill_pos(a.pos, dev=dev, max_len=a.max_seqlen, span=span, position_buckets=position_buckets,
                max_relative_distance=max_relative_distance, pos_key=pk, pos_query=pq,
                c2p_strip=strips[0], p2c_strip=strips[1], varlen=True, keep=keep)
-    with torch.cuda.device(dev):
-        _lib.check(_lib.load().tdb_attn_fwd_varlen(C.byref(a), L.stream_of(dev)))
-    return o
+    keep += [t for t in (strips[0], strips[1], pk, pq) if t is not None]
+    return L.PreparedLaunch(_lib.load().tdb_attn_fwd_varlen, a, o, keep, dev)
 
 
 class FlashAttentionDisentangled(torch.autograd.Function):
@@ -87,9 +88,9 @@ class FlashAttentionDisentangled(torch.autograd.Function):
     @staticmethod
     def forward(ctx, q, k, v, q_pos, k_pos, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, causal,
                 sm_scale, position_buckets, max_relative_distance, pos_key_layer, pos_query_layer, force_generic):
-        return _forward(q, k, v, q_pos, k_pos, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, causal,
-                        sm_scale, position_buckets, max_relative_distance, pos_key_layer, pos_query_layer,
-                        force_generic)
+        return prepare(q, k, v, q_pos, k_pos, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, causal,
+                       sm_scale, position_buckets, max_relative_distance, pos_key_layer=pos_key_layer,
+                       pos_query_layer=pos_query_layer, force_generic=force_generic).launch()
 
     @staticmethod
     def backward(ctx, grad_output):
