@@ -33,10 +33,25 @@ typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 
 #define TDB_LDS(T, p) ((__attribute__((address_space(3))) T*)(p))
 
+// Phase timing for development builds (-DTDB_TIMING): one wave accumulates cycle counts per phase.
+#ifdef TDB_TIMING
+__device__ long long tdb_timing[16];
+#define TDB_T0() long long tdb_t = clock64(); const bool tdb_on = blockIdx.x == 7 && blockIdx.y == 3 && threadIdx.x == 64
+#define TDB_TICK(k)                                        \
+    do {                                                   \
+        const long long n_ = clock64();                    \
+        if (tdb_on) tdb_timing[k] += n_ - tdb_t;           \
+        tdb_t = n_;                                        \
+    } while (0)
+#else
+#define TDB_T0() do {} while (0)
+#define TDB_TICK(k) do {} while (0)
+#endif
+
 constexpr int BM = TDB_MFMA_TILE;   // query rows per workgroup
 constexpr int BN = 64;              // keys per step
 constexpr int D = 64;
-constexpr int WIN = BM + BN;        // staged window rows (one more than the 191 positions in use)
+constexpr int WIN = BM + BN;        // ring of staged window rows (one more than the 191 positions in use)
 constexpr int RS = 72;              // LDS row stride (elements) of 64-wide bf16 rows: 144 B, conflict-free b128
 constexpr int CS = 100;             // row stride (floats) of the per-wave c2p scratch [32][96 used]
 constexpr int PS = 196;             // row stride of the p2c scratch           [64][192 used]
@@ -152,38 +167,89 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const TdbKernelParams p)
     const int lut_max = 2 * p.lut_half;
     const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
 
-    for (int j0 = 0; j0 < len; j0 += BN) {
-        __syncthreads();   // everyone is done reading the previous step's tiles
-        // ---- stage K, V (rows past the sequence end become zeros) -------------------------------------
+    // ---- staging ---------------------------------------------------------------------------------------------
+    // Key step s covers keys 64s .. 64s+63 and needs relative positions B_s .. B_s+190, B_s = row0 - 64s - 63.
+    // The rows K_r[delta(r)] / Q_r[delta(r)] of that window live in a 192-row ring: going to the next step the
+    // window slides down by 64, so only its 64 lowest positions are fetched and they overwrite the 64 highest
+    // of the previous step.  Window row x of step s sits in ring slot (x + off_s) mod 192, off_s = (128*s) mod 192.
+    // Everything a step needs from global memory is fetched one step ahead into registers (delta values two
+    // steps ahead) and written to LDS between two barriers.
+    constexpr bool HAS_POS = HAS_C2P || HAS_P2C;
+    const int nsteps = (len + BN - 1) / BN;
+    const int srow = tid >> 3, sch = tid & 7;              // this thread stages rows srow, srow+32 (chunk sch)
+    auto delta_of = [&](int r) { return p.lut[min(max(r + p.lut_half, 0), lut_max)]; };
+
+    u32x4 pre_k[2], pre_v[2], pre_kr[2], pre_qr[2];
+    int dl_next[2] = {0, 0};
+    auto fetch_step = [&](int s) {       // global -> registers for key step s (its keys and its 64 new window rows)
 #pragma unroll
         for (int n = 0; n < 2; ++n) {
-            const int idx = tid + 256 * n, r = idx >> 3, ch = idx & 7;
-            u32x4 kk = {0, 0, 0, 0}, vv = {0, 0, 0, 0};
-            if (j0 + r < len) {
-                kk = *reinterpret_cast<const u32x4*>(K + int64_t(j0 + r) * p.ks_l + ch * 8);
-                vv = *reinterpret_cast<const u32x4*>(V + int64_t(j0 + r) * p.vs_l + ch * 8);
+            const int j = BN * s + srow + 32 * n;
+            pre_k[n] = u32x4{0, 0, 0, 0};
+            pre_v[n] = u32x4{0, 0, 0, 0};
+            if (j < len) {
+                pre_k[n] = *reinterpret_cast<const u32x4*>(K + int64_t(j) * p.ks_l + sch * 8);
+                pre_v[n] = *reinterpret_cast<const u32x4*>(V + int64_t(j) * p.vs_l + sch * 8);
             }
-            *reinterpret_cast<u32x4*>(&sm.k[r * RS + ch * 8]) = kk;
-            *reinterpret_cast<u32x4*>(&sm.v[r * RS + ch * 8]) = vv;
+            if (HAS_C2P) pre_kr[n] = *reinterpret_cast<const u32x4*>(PK + int64_t(dl_next[n]) * p.pks_r + sch * 8);
+            if (HAS_P2C) pre_qr[n] = *reinterpret_cast<const u32x4*>(PQ + int64_t(dl_next[n]) * p.pqs_r + sch * 8);
         }
-        // ---- stage the position window: row x holds relative position r = row0 - j0 - 63 + x ----------
-        if (HAS_C2P || HAS_P2C) {
-            const int rbase = row0 - j0 - (BN - 1);
+    };
+    auto fetch_delta = [&](int s) {      // delta of the 64 new window rows of key step s
+        if (HAS_POS) {
 #pragma unroll
-            for (int n = 0; n < WIN * 8 / 256; ++n) {
-                const int idx = tid + 256 * n, x = idx >> 3, ch = idx & 7;
-                const int li = min(max(rbase + x + p.lut_half, 0), lut_max);
-                const int dl = p.lut[li];
-                if (HAS_C2P)
-                    *reinterpret_cast<u32x4*>(&sm.kr[x * RS + ch * 8]) =
-                        *reinterpret_cast<const u32x4*>(PK + int64_t(dl) * p.pks_r + ch * 8);
-                if (HAS_P2C)
-                    *reinterpret_cast<u32x4*>(&sm.qr[x * RS + ch * 8]) =
-                        *reinterpret_cast<const u32x4*>(PQ + int64_t(dl) * p.pqs_r + ch * 8);
-            }
+            for (int n = 0; n < 2; ++n) dl_next[n] = delta_of(row0 - BN * s - (BN - 1) + srow + 32 * n);
         }
-        __syncthreads();
+    };
+    auto store_step = [&](int off) {     // registers -> LDS
+#pragma unroll
+        for (int n = 0; n < 2; ++n) {
+            const int r = srow + 32 * n;
+            *reinterpret_cast<u32x4*>(&sm.k[r * RS + sch * 8]) = pre_k[n];
+            *reinterpret_cast<u32x4*>(&sm.v[r * RS + sch * 8]) = pre_v[n];
+            if (HAS_C2P) *reinterpret_cast<u32x4*>(&sm.kr[(off + r) * RS + sch * 8]) = pre_kr[n];
+            if (HAS_P2C) *reinterpret_cast<u32x4*>(&sm.qr[(off + r) * RS + sch * 8]) = pre_qr[n];
+        }
+    };
 
+    // prologue: whole window of step 0 (slots 0..191), keys of step 0
+    if (HAS_POS) {
+#pragma unroll
+        for (int n = 0; n < WIN * 8 / 256; ++n) {
+            const int x = srow + 32 * n;
+            const int dl = delta_of(row0 - (BN - 1) + x);
+            if (HAS_C2P)
+                *reinterpret_cast<u32x4*>(&sm.kr[x * RS + sch * 8]) = *reinterpret_cast<const u32x4*>(PK + int64_t(dl) * p.pks_r + sch * 8);
+            if (HAS_P2C)
+                *reinterpret_cast<u32x4*>(&sm.qr[x * RS + sch * 8]) = *reinterpret_cast<const u32x4*>(PQ + int64_t(dl) * p.pqs_r + sch * 8);
+        }
+    }
+#pragma unroll
+    for (int n = 0; n < 2; ++n) {
+        const int r = srow + 32 * n;
+        u32x4 kk = {0, 0, 0, 0}, vv = {0, 0, 0, 0};
+        if (r < len) {
+            kk = *reinterpret_cast<const u32x4*>(K + int64_t(r) * p.ks_l + sch * 8);
+            vv = *reinterpret_cast<const u32x4*>(V + int64_t(r) * p.vs_l + sch * 8);
+        }
+        *reinterpret_cast<u32x4*>(&sm.k[r * RS + sch * 8]) = kk;
+        *reinterpret_cast<u32x4*>(&sm.v[r * RS + sch * 8]) = vv;
+    }
+    fetch_delta(1);
+    __syncthreads();
+    if (nsteps > 1) {
+        fetch_step(1);
+        fetch_delta(2);
+    }
+
+    int off = 0;                          // ring slot of window row 0 of the current step
+    TDB_T0();
+    for (int s = 0; s < nsteps; ++s) {
+        const int j0 = BN * s;
+        // ring rows of the position tiles this wave reads as MFMA A operands
+        auto ring = [&](int x) { const int t = x + off; return t >= WIN ? t - WIN : t; };
+
+        TDB_TICK(0);
         // ---- K fragments: A operand of S^T = K.Q^T and B operand of P'^T = Q_r'.K^T ---------------------
         bf16x8 kf[2][4];
 #pragma unroll
@@ -200,7 +266,7 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const TdbKernelParams p)
                 for (int e = 0; e < 16; ++e) acc[e] = 0.f;
 #pragma unroll
                 for (int c = 0; c < 4; ++c)
-                    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lds_frag(sm.kr, 32 * w + 32 * rt + il, 16 * c + 8 * hh),
+                    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lds_frag(sm.kr, ring(32 * w + 32 * rt + il), 16 * c + 8 * hh),
                                                                   qb[c], acc, 0, 0, 0);
 #pragma unroll
                 for (int a = 0; a < 4; ++a)
@@ -208,6 +274,7 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const TdbKernelParams p)
                         float4{acc[4 * a], acc[4 * a + 1], acc[4 * a + 2], acc[4 * a + 3]};
             }
         }
+        TDB_TICK(1);
         // ---- p2c: P'^T[r, j] for the whole window (6 x 2 tiles): wave w takes position tile w against both
         //      key tiles, then one tile of position tiles 4..5; to LDS as P'[j][r''] -----------------------------
         if (HAS_P2C) {
@@ -217,7 +284,7 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const TdbKernelParams p)
                 for (int e = 0; e < 16; ++e) acc[e] = 0.f;
 #pragma unroll
                 for (int c = 0; c < 4; ++c)
-                    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lds_frag(sm.qr, 32 * rt + il, 16 * c + 8 * hh), kb[c], acc, 0, 0, 0);
+                    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lds_frag(sm.qr, ring(32 * rt + il), 16 * c + 8 * hh), kb[c], acc, 0, 0, 0);
 #pragma unroll
                 for (int a = 0; a < 4; ++a)
                     *reinterpret_cast<u32x2*>(&sm.p[(32 * jt + il) * PS + 32 * rt + 8 * a + 4 * hh]) =
@@ -228,7 +295,9 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const TdbKernelParams p)
             if (w & 1) p2c_tile(4 + (w >> 1), 1, kf[1]);
             else p2c_tile(4 + (w >> 1), 0, kf[0]);
         }
+        TDB_TICK(2);
         __syncthreads();
+        TDB_TICK(3);
 
         // ---- S^T = K.Q^T + position terms.  Element (jj, i) of the tile takes C'[i][i-jj+63] (fp32, gathered
         //      straight into the accumulator the MFMA then adds onto) and P'[jj][32w+i-jj+63] (bf16) ------------
@@ -269,6 +338,7 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const TdbKernelParams p)
                     s_acc[jt][e] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, g[e]), ones, s_acc[jt][e], false);
             }
         }
+        TDB_TICK(4);
         // ---- mask keys past the end of the sequence (last step only) ------------------------------------------
         if (j0 + BN > len) {
 #pragma unroll
@@ -311,6 +381,7 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const TdbKernelParams p)
 #pragma unroll
             for (int e = 0; e < 16; ++e) o_acc[t][e] *= alpha;
 
+        TDB_TICK(5);
         // ---- O^T += V^T.P^T; V^T fragments come from row-major V through the transposing LDS read ----------
         {
             const int g = l >> 4, ll = l & 15;
@@ -329,6 +400,20 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const TdbKernelParams p)
                         o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, both), pb[jt][c], o_acc[dt], 0, 0, 0);
                     }
         }
+
+        TDB_TICK(6);
+        // ---- hand the prefetched next step to LDS and start fetching the one after -------------------------
+        if (s + 1 < nsteps) {
+            off = off >= BN ? off - BN : off + WIN - BN;
+            __syncthreads();              // every wave is done with this step's tiles
+            store_step(off);
+            __syncthreads();
+            if (s + 2 < nsteps) {
+                fetch_step(s + 2);
+                fetch_delta(s + 3);
+            }
+        }
+        TDB_TICK(7);
     }
 
     // ---- epilogue: normalise and store O[i][d]; lane holds d = 32*dt + 8*a + 4*hh + 0..3 of query row il ------
