@@ -167,13 +167,19 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const TdbKernelParams p)
     const int lut_max = 2 * p.lut_half;
     const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
 
-    // ---- staging ---------------------------------------------------------------------------------------------
+    // ---- pipeline ----------------------------------------------------------------------------------------------
     // Key step s covers keys 64s .. 64s+63 and needs relative positions B_s .. B_s+190, B_s = row0 - 64s - 63.
     // The rows K_r[delta(r)] / Q_r[delta(r)] of that window live in a 192-row ring: going to the next step the
     // window slides down by 64, so only its 64 lowest positions are fetched and they overwrite the 64 highest
     // of the previous step.  Window row x of step s sits in ring slot (x + off_s) mod 192, off_s = (128*s) mod 192.
-    // Everything a step needs from global memory is fetched one step ahead into registers (delta values two
-    // steps ahead) and written to LDS between two barriers.
+    //
+    // Each step has two halves separated by workgroup barriers:
+    //   A  read this step's position terms out of the C'/P' scratch (into the score accumulators) and hand the
+    //      register-prefetched global data to LDS: keys of step s+1, values of step s, 64 window rows of step s+1;
+    //   B  matrix work: S^T(s) = K.Q^T on top of the position terms, then the position products C', P' of step
+    //      s+1 into the now free scratch, softmax(s) on the vector ALUs, P.V(s); global fetches for half A of the
+    //      next step are issued at the start of B.
+    // The K fragments of step s+1 are read from LDS in half B (for P'(s+1)) and stay in registers for S^T(s+1).
     constexpr bool HAS_POS = HAS_C2P || HAS_P2C;
     const int nsteps = (len + BN - 1) / BN;
     const int srow = tid >> 3, sch = tid & 7;              // this thread stages rows srow, srow+32 (chunk sch)
@@ -181,16 +187,15 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const TdbKernelParams p)
 
     u32x4 pre_k[2], pre_v[2], pre_kr[2], pre_qr[2];
     int dl_next[2] = {0, 0};
-    auto fetch_step = [&](int s) {       // global -> registers for key step s (its keys and its 64 new window rows)
+    // global -> registers: key rows of step sk, value rows of step sv, the 64 new window rows whose delta is in
+    // dl_next.  Rows past the end of the sequence re-read its last row (finite data; those keys are masked and
+    // get probability 0), so no lane is predicated off and the code stays branch-free.
+    auto fetch = [&](int sk, int sv) {
 #pragma unroll
         for (int n = 0; n < 2; ++n) {
-            const int j = BN * s + srow + 32 * n;
-            pre_k[n] = u32x4{0, 0, 0, 0};
-            pre_v[n] = u32x4{0, 0, 0, 0};
-            if (j < len) {
-                pre_k[n] = *reinterpret_cast<const u32x4*>(K + int64_t(j) * p.ks_l + sch * 8);
-                pre_v[n] = *reinterpret_cast<const u32x4*>(V + int64_t(j) * p.vs_l + sch * 8);
-            }
+            const int jk = min(BN * sk + srow + 32 * n, len - 1), jv = min(BN * sv + srow + 32 * n, len - 1);
+            pre_k[n] = *reinterpret_cast<const u32x4*>(K + int64_t(jk) * p.ks_l + sch * 8);
+            pre_v[n] = *reinterpret_cast<const u32x4*>(V + int64_t(jv) * p.vs_l + sch * 8);
             if (HAS_C2P) pre_kr[n] = *reinterpret_cast<const u32x4*>(PK + int64_t(dl_next[n]) * p.pks_r + sch * 8);
             if (HAS_P2C) pre_qr[n] = *reinterpret_cast<const u32x4*>(PQ + int64_t(dl_next[n]) * p.pqs_r + sch * 8);
         }
@@ -201,7 +206,7 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const TdbKernelParams p)
             for (int n = 0; n < 2; ++n) dl_next[n] = delta_of(row0 - BN * s - (BN - 1) + srow + 32 * n);
         }
     };
-    auto store_step = [&](int off) {     // registers -> LDS
+    auto store = [&](int off) {          // registers -> LDS
 #pragma unroll
         for (int n = 0; n < 2; ++n) {
             const int r = srow + 32 * n;
@@ -212,7 +217,88 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const TdbKernelParams p)
         }
     };
 
-    // prologue: whole window of step 0 (slots 0..191), keys of step 0
+    // K fragments: A operand of S^T = K.Q^T, B operand of P'^T = Q_r'.K^T
+    bf16x8 kf[2][4];
+    auto load_kf = [&](bf16x8 (&dst)[2][4]) {
+#pragma unroll
+        for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) dst[jt][c] = lds_frag(sm.k, 32 * jt + il, 16 * c + 8 * hh);
+    };
+    const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    const bool odd_wave = (w & 1) != 0;
+    // LDS reads of every A fragment the position products of one step need: c2p position tiles 0..2 of this wave's
+    // sub-window (fr[0..2]) and p2c position tiles w and 4 + w/2 of the workgroup window (fr[3], fr[4]).
+    auto load_pos_frags = [&](int off, bf16x8 (&fr)[5][4]) {
+        auto ring = [&](int x) { const int t = x + off; return t >= WIN ? t - WIN : t; };
+        if (HAS_C2P) {
+#pragma unroll
+            for (int rt = 0; rt < 3; ++rt) {
+                const int row = ring(32 * w + 32 * rt + il);
+#pragma unroll
+                for (int c = 0; c < 4; ++c) fr[rt][c] = lds_frag(sm.kr, row, 16 * c + 8 * hh);
+            }
+        }
+        if (HAS_P2C) {
+            const int row3 = ring(32 * w + il), row4 = ring(32 * (4 + (w >> 1)) + il);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                fr[3][c] = lds_frag(sm.qr, row3, 16 * c + 8 * hh);
+                fr[4][c] = lds_frag(sm.qr, row4, 16 * c + 8 * hh);
+            }
+        }
+    };
+    // Position products of one key step from fragments already in registers, into the scratch:
+    //   c2p  C'^T[r, i] = K_r'[r].Q_i over this wave's 96-position sub-window, stored as fp32 C'[i][r'];
+    //   p2c  P'^T[r, j] = Q_r'[r].K_j over the whole window (6 x 2 tiles): wave w takes position tile w against both
+    //        key tiles and tile (4 + w/2, w&1); stored as bf16 P'[j][r''].
+    auto pos_products = [&](const bf16x8 (&fr)[5][4], const bf16x8 (&kn)[2][4]) {
+        auto chain = [&](const bf16x8 (&a)[4], const bf16x8 (&bb)[4]) {
+            f32x16 acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], bb[0], zero16, 0, 0, 0);
+#pragma unroll
+            for (int c = 1; c < 4; ++c) acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[c], bb[c], acc, 0, 0, 0);
+            return acc;
+        };
+        auto put_c = [&](int rt, const f32x16& acc) {
+#pragma unroll
+            for (int a = 0; a < 4; ++a)
+                *reinterpret_cast<float4*>(&sm.c[w][il * CS + 32 * rt + 8 * a + 4 * hh]) =
+                    float4{acc[4 * a], acc[4 * a + 1], acc[4 * a + 2], acc[4 * a + 3]};
+        };
+        auto put_p = [&](int rt, int jt, const f32x16& acc) {
+#pragma unroll
+            for (int a = 0; a < 4; ++a)
+                *reinterpret_cast<u32x2*>(&sm.p[(32 * jt + il) * PS + 32 * rt + 8 * a + 4 * hh]) =
+                    pack4(acc[4 * a], acc[4 * a + 1], acc[4 * a + 2], acc[4 * a + 3]);
+        };
+        if (HAS_C2P) {
+            const f32x16 a0 = chain(fr[0], qb);
+            const f32x16 a1 = chain(fr[1], qb);
+            put_c(0, a0);
+            const f32x16 a2 = chain(fr[2], qb);
+            put_c(1, a1);
+            put_c(2, a2);
+        }
+        if (HAS_P2C) {
+            bf16x8 kx[4];                 // key tile (w & 1), chosen without indexing registers
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const u32x4 x0 = __builtin_bit_cast(u32x4, kn[0][c]), x1 = __builtin_bit_cast(u32x4, kn[1][c]);
+                u32x4 r;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) r[e] = odd_wave ? x1[e] : x0[e];
+                kx[c] = __builtin_bit_cast(bf16x8, r);
+            }
+            const f32x16 a0 = chain(fr[3], kn[0]);
+            const f32x16 a1 = chain(fr[3], kn[1]);
+            put_p(w, 0, a0);
+            const f32x16 a2 = chain(fr[4], kx);
+            put_p(w, 1, a1);
+            put_p(4 + (w >> 1), w & 1, a2);
+        }
+    };
+
+    // prologue: keys and whole window of step 0 to LDS, position products of step 0, prefetch for half A of step 0
     if (HAS_POS) {
 #pragma unroll
         for (int n = 0; n < WIN * 8 / 256; ++n) {
@@ -227,80 +313,29 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const TdbKernelParams p)
 #pragma unroll
     for (int n = 0; n < 2; ++n) {
         const int r = srow + 32 * n;
-        u32x4 kk = {0, 0, 0, 0}, vv = {0, 0, 0, 0};
-        if (r < len) {
-            kk = *reinterpret_cast<const u32x4*>(K + int64_t(r) * p.ks_l + sch * 8);
-            vv = *reinterpret_cast<const u32x4*>(V + int64_t(r) * p.vs_l + sch * 8);
-        }
-        *reinterpret_cast<u32x4*>(&sm.k[r * RS + sch * 8]) = kk;
-        *reinterpret_cast<u32x4*>(&sm.v[r * RS + sch * 8]) = vv;
+        *reinterpret_cast<u32x4*>(&sm.k[r * RS + sch * 8]) =
+            *reinterpret_cast<const u32x4*>(K + int64_t(min(r, len - 1)) * p.ks_l + sch * 8);
     }
     fetch_delta(1);
     __syncthreads();
-    if (nsteps > 1) {
-        fetch_step(1);
-        fetch_delta(2);
+    fetch(1, 0);
+    fetch_delta(2);
+    load_kf(kf);
+    {
+        bf16x8 fr[5][4];
+        load_pos_frags(0, fr);
+        pos_products(fr, kf);
     }
 
-    int off = 0;                          // ring slot of window row 0 of the current step
     TDB_T0();
-    for (int s = 0; s < nsteps; ++s) {
-        const int j0 = BN * s;
-        // ring rows of the position tiles this wave reads as MFMA A operands
-        auto ring = [&](int x) { const int t = x + off; return t >= WIN ? t - WIN : t; };
-
+    // One key step.  MASKED: the step reaches past the end of the sequence (only the last step can).
+    auto key_step = [&](int s, int off, int off_next, auto masked_tag) {
+        constexpr bool MASKED = decltype(masked_tag)::value;
+        __syncthreads();                  // scratch of step s complete; every wave holds its K fragments of step s
         TDB_TICK(0);
-        // ---- K fragments: A operand of S^T = K.Q^T and B operand of P'^T = Q_r'.K^T ---------------------
-        bf16x8 kf[2][4];
-#pragma unroll
-        for (int jt = 0; jt < 2; ++jt)
-#pragma unroll
-            for (int c = 0; c < 4; ++c) kf[jt][c] = lds_frag(sm.k, 32 * jt + il, 16 * c + 8 * hh);
 
-        // ---- c2p: C'^T[r, i] over this wave's 96-position sub-window, to LDS as C'[i][r'] --------------
-        if (HAS_C2P) {
-#pragma unroll
-            for (int rt = 0; rt < 3; ++rt) {
-                f32x16 acc;
-#pragma unroll
-                for (int e = 0; e < 16; ++e) acc[e] = 0.f;
-#pragma unroll
-                for (int c = 0; c < 4; ++c)
-                    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lds_frag(sm.kr, ring(32 * w + 32 * rt + il), 16 * c + 8 * hh),
-                                                                  qb[c], acc, 0, 0, 0);
-#pragma unroll
-                for (int a = 0; a < 4; ++a)
-                    *reinterpret_cast<float4*>(&sm.c[w][il * CS + 32 * rt + 8 * a + 4 * hh]) =
-                        float4{acc[4 * a], acc[4 * a + 1], acc[4 * a + 2], acc[4 * a + 3]};
-            }
-        }
-        TDB_TICK(1);
-        // ---- p2c: P'^T[r, j] for the whole window (6 x 2 tiles): wave w takes position tile w against both
-        //      key tiles, then one tile of position tiles 4..5; to LDS as P'[j][r''] -----------------------------
-        if (HAS_P2C) {
-            auto p2c_tile = [&](int rt, int jt, const bf16x8 (&kb)[4]) {
-                f32x16 acc;
-#pragma unroll
-                for (int e = 0; e < 16; ++e) acc[e] = 0.f;
-#pragma unroll
-                for (int c = 0; c < 4; ++c)
-                    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lds_frag(sm.qr, ring(32 * rt + il), 16 * c + 8 * hh), kb[c], acc, 0, 0, 0);
-#pragma unroll
-                for (int a = 0; a < 4; ++a)
-                    *reinterpret_cast<u32x2*>(&sm.p[(32 * jt + il) * PS + 32 * rt + 8 * a + 4 * hh]) =
-                        pack4(acc[4 * a], acc[4 * a + 1], acc[4 * a + 2], acc[4 * a + 3]);
-            };
-            p2c_tile(w, 0, kf[0]);
-            p2c_tile(w, 1, kf[1]);
-            if (w & 1) p2c_tile(4 + (w >> 1), 1, kf[1]);
-            else p2c_tile(4 + (w >> 1), 0, kf[0]);
-        }
-        TDB_TICK(2);
-        __syncthreads();
-        TDB_TICK(3);
-
-        // ---- S^T = K.Q^T + position terms.  Element (jj, i) of the tile takes C'[i][i-jj+63] (fp32, gathered
-        //      straight into the accumulator the MFMA then adds onto) and P'[jj][32w+i-jj+63] (bf16) ------------
+        // ---- half A: position terms of step s out of the scratch.  Element (jj, i) of the score tile takes
+        //      C'[i][i-jj+63] (fp32, straight into the accumulator) and P'[jj][32w+i-jj+63] (bf16) ----------------
         f32x16 s_acc[2];
         if (HAS_C2P) {
             // float index of element e of key tile jt:  il*CS + il + 63 - 4*hh - jc,  jc = 32*jt + 8*(e>>2) + (e&3) <= 59
@@ -312,51 +347,80 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const TdbKernelParams p)
                 s_acc[jt][e] = t.x;
                 s_acc[jt][e + 1] = t.y;
             });
-            lds_wait(s_acc[0], s_acc[1]);
+            if (!HAS_P2C) lds_wait(s_acc[0], s_acc[1]);
         } else {
+            s_acc[0] = zero16;
+            s_acc[1] = zero16;
+        }
+        if (HAS_P2C) {
+            const uint32_t paddr = lds_addr(&sm.p[32 * w + il + 63 + 4 * hh * (PS - 1)]);
+            uint32_t g[2][16];
+            static_for<32>([&](auto ec) {
+                constexpr int jt = decltype(ec)::value >> 4, e = decltype(ec)::value & 15;
+                constexpr int jc = 32 * jt + 8 * (e >> 2) + (e & 3);
+                g[jt][e] = lds_read_u16<2 * jc * (PS - 1)>(paddr);
+            });
+            lds_wait(g[0]);
+            lds_wait(g[1]);
+            lds_wait(s_acc[0], s_acc[1]);
 #pragma unroll
             for (int jt = 0; jt < 2; ++jt)
 #pragma unroll
-                for (int e = 0; e < 16; ++e) s_acc[jt][e] = 0.f;
-        }
-#pragma unroll
-        for (int jt = 0; jt < 2; ++jt)
-#pragma unroll
-            for (int c = 0; c < 4; ++c) s_acc[jt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[jt][c], qb[c], s_acc[jt], 0, 0, 0);
-        if (HAS_P2C) {
-            const uint32_t paddr = lds_addr(&sm.p[32 * w + il + 63 + 4 * hh * (PS - 1)]);
-#pragma unroll
-            for (int jt = 0; jt < 2; ++jt) {
-                uint32_t g[16];
-                static_for<16>([&](auto ec) {
-                    constexpr int e = decltype(ec)::value, jc0 = 8 * (e >> 2) + (e & 3);
-                    g[e] = jt == 0 ? lds_read_u16<2 * jc0 * (PS - 1)>(paddr) : lds_read_u16<2 * (32 + jc0) * (PS - 1)>(paddr);
-                });
-                lds_wait(g);
-#pragma unroll
                 for (int e = 0; e < 16; ++e)   // bf16 pair (value, 0) . (1, 1) + acc
-                    s_acc[jt][e] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, g[e]), ones, s_acc[jt][e], false);
-            }
+                    s_acc[jt][e] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, g[jt][e]), ones, s_acc[jt][e], false);
         }
-        TDB_TICK(4);
-        // ---- mask keys past the end of the sequence (last step only) ------------------------------------------
-        if (j0 + BN > len) {
+        store(off_next);                  // keys of step s+1, values of step s, new window rows of step s+1
+        TDB_TICK(1);
+        __syncthreads();                  // scratch is free again; the staged tiles are visible
+        TDB_TICK(2);
+
+        // ---- half B (one basic block, so that matrix and vector work can be interleaved) ------------------------
+        fetch(s + 2, s + 1);
+        fetch_delta(s + 3);
+        bf16x8 kn[2][4], fr[5][4];
+        load_kf(kn);                      // K fragments of step s+1
+        load_pos_frags(off_next, fr);
+        // V^T fragments through the transposing LDS read: lane provides the address of 4 dims of one key
+        bf16x8 vf[2][2][2];               // [key tile][16-key chunk][dim tile]
+        {
+            const int g = l >> 4, ll = l & 15;
+            const uint16_t* vbase = &sm.v[((ll >> 2) + 4 * (g >> 1)) * RS + 16 * (g & 1) + 4 * (ll & 3)];
+#pragma unroll
+            for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+                for (int c = 0; c < 2; ++c)
+#pragma unroll
+                    for (int dt = 0; dt < 2; ++dt) {
+                        const uint16_t* src = vbase + (32 * jt + 16 * c) * RS + 32 * dt;
+                        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(TDB_LDS(s16x4, src));
+                        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(TDB_LDS(s16x4, src + 8 * RS));
+                        const __attribute__((ext_vector_type(8))) short both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                        vf[jt][c][dt] = __builtin_bit_cast(bf16x8, both);
+                    }
+        }
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+#pragma unroll
+            for (int jt = 0; jt < 2; ++jt) s_acc[jt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[jt][c], qb[c], s_acc[jt], 0, 0, 0);
+        pos_products(fr, kn);             // of step s+1 (harmless left-over work in the last step)
+        TDB_TICK(3);
+        if (MASKED) {
 #pragma unroll
             for (int jt = 0; jt < 2; ++jt)
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
-                    const int j = j0 + 32 * jt + 8 * (e >> 2) + 4 * hh + (e & 3);
+                    const int j = BN * s + 32 * jt + 8 * (e >> 2) + 4 * hh + (e & 3);
                     if (j >= len) s_acc[jt][e] = -INFINITY;
                 }
         }
-        // ---- streaming softmax: this lane holds 32 of the 64 keys of query row il, lane^32 the others -------
+        // streaming softmax: this lane holds 32 of the 64 keys of query row il, lane^32 the others
         float mx = s_acc[0][0];
 #pragma unroll
         for (int jt = 0; jt < 2; ++jt)
 #pragma unroll
             for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s_acc[jt][e]);
         mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float m_new = fmaxf(m_run, mx);          // finite: key j0 < len is never masked
+        const float m_new = fmaxf(m_run, mx);          // finite: key 64s < len is never masked
         const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * c_exp);
         const float mc = m_new * c_exp;
         m_run = m_new;
@@ -380,41 +444,30 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const TdbKernelParams p)
         for (int t = 0; t < 2; ++t)
 #pragma unroll
             for (int e = 0; e < 16; ++e) o_acc[t][e] *= alpha;
-
+        TDB_TICK(4);
+        // O^T += V^T.P^T
+#pragma unroll
+        for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+            for (int c = 0; c < 2; ++c)
+#pragma unroll
+                for (int dt = 0; dt < 2; ++dt)
+                    o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[jt][c][dt], pb[jt][c], o_acc[dt], 0, 0, 0);
+#pragma unroll
+        for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) kf[jt][c] = kn[jt][c];
         TDB_TICK(5);
-        // ---- O^T += V^T.P^T; V^T fragments come from row-major V through the transposing LDS read ----------
-        {
-            const int g = l >> 4, ll = l & 15;
-            // source address of this lane inside a 4-key x 16-dim block: row (ll>>2), 4 dims at 4*(ll&3)
-            const uint16_t* vbase = &sm.v[((ll >> 2) + 4 * (g >> 1)) * RS + 16 * (g & 1) + 4 * (ll & 3)];
-#pragma unroll
-            for (int jt = 0; jt < 2; ++jt)
-#pragma unroll
-                for (int c = 0; c < 2; ++c)
-#pragma unroll
-                    for (int dt = 0; dt < 2; ++dt) {
-                        const uint16_t* src = vbase + (32 * jt + 16 * c) * RS + 32 * dt;
-                        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(TDB_LDS(s16x4, src));
-                        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(TDB_LDS(s16x4, src + 8 * RS));
-                        const __attribute__((ext_vector_type(8))) short both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                        o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, both), pb[jt][c], o_acc[dt], 0, 0, 0);
-                    }
-        }
+    };
 
-        TDB_TICK(6);
-        // ---- hand the prefetched next step to LDS and start fetching the one after -------------------------
-        if (s + 1 < nsteps) {
-            off = off >= BN ? off - BN : off + WIN - BN;
-            __syncthreads();              // every wave is done with this step's tiles
-            store_step(off);
-            __syncthreads();
-            if (s + 2 < nsteps) {
-                fetch_step(s + 2);
-                fetch_delta(s + 3);
-            }
-        }
-        TDB_TICK(7);
+    int off = 0;                          // ring slot of window row 0 of the current step
+    const int nfull = len / BN;           // steps that need no key mask
+    for (int s = 0; s < nfull; ++s) {
+        const int off_next = off >= BN ? off - BN : off + WIN - BN;
+        key_step(s, off, off_next, std::false_type{});
+        off = off_next;
     }
+    if (nfull < nsteps) key_step(nfull, off, off >= BN ? off - BN : off + WIN - BN, std::true_type{});
 
     // ---- epilogue: normalise and store O[i][d]; lane holds d = 32*dt + 8*a + 4*hh + 0..3 of query row il ------
     const float l_tot = l_run + __shfl_xor(l_run, 32);
