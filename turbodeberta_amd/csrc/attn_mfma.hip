@@ -187,17 +187,34 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const TdbKernelParams p)
 
     u32x4 pre_k[2], pre_v[2], pre_kr[2], pre_qr[2];
     int dl_next[2] = {0, 0};
-    // global -> registers: key rows of step sk, value rows of step sv, the 64 new window rows whose delta is in
-    // dl_next.  Rows past the end of the sequence re-read its last row (finite data; those keys are masked and
-    // get probability 0), so no lane is predicated off and the code stays branch-free.
+    // global -> registers through buffer loads: key rows of step sk, value rows of step sv, the 64 new window rows
+    // whose delta is in dl_next.  The buffer of a step starts at its first row and ends with the last row of the
+    // sequence, so rows past the end come back as zeros (hardware range check) with no lane predicated off, and the
+    // only per-load address arithmetic left is scalar.
+    const int ks_b = int(p.ks_l) * 2, vs_b = int(p.vs_l) * 2, pks_b = int(p.pks_r) * 2, pqs_b = int(p.pqs_r) * 2;
+    int kvoff[2], vvoff[2];               // byte offsets of this thread's two rows inside a step's buffer
+#pragma unroll
+    for (int n = 0; n < 2; ++n) {
+        kvoff[n] = (srow + 32 * n) * ks_b + sch * 16;
+        vvoff[n] = (srow + 32 * n) * vs_b + sch * 16;
+    }
+    constexpr int RSRC_FLAGS = 0x00020000;   // raw buffer, 32-bit data format
+    const __amdgpu_buffer_rsrc_t pk_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(HAS_C2P ? PK : K), 0, HAS_C2P ? (2 * p.span - 1) * pks_b + 128 : 0, RSRC_FLAGS);
+    const __amdgpu_buffer_rsrc_t pq_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(HAS_P2C ? PQ : K), 0, HAS_P2C ? (2 * p.span - 1) * pqs_b + 128 : 0, RSRC_FLAGS);
     auto fetch = [&](int sk, int sv) {
+        const int kleft = len - BN * sk, vleft = len - BN * sv;      // rows of the sequence from the step's first row on
+        const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<uint16_t*>(K) + int64_t(BN * sk) * p.ks_l, 0, kleft > 0 ? (kleft - 1) * ks_b + 128 : 0, RSRC_FLAGS);
+        const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<uint16_t*>(V) + int64_t(BN * sv) * p.vs_l, 0, vleft > 0 ? (vleft - 1) * vs_b + 128 : 0, RSRC_FLAGS);
 #pragma unroll
         for (int n = 0; n < 2; ++n) {
-            const int jk = min(BN * sk + srow + 32 * n, len - 1), jv = min(BN * sv + srow + 32 * n, len - 1);
-            pre_k[n] = *reinterpret_cast<const u32x4*>(K + int64_t(jk) * p.ks_l + sch * 8);
-            pre_v[n] = *reinterpret_cast<const u32x4*>(V + int64_t(jv) * p.vs_l + sch * 8);
-            if (HAS_C2P) pre_kr[n] = *reinterpret_cast<const u32x4*>(PK + int64_t(dl_next[n]) * p.pks_r + sch * 8);
-            if (HAS_P2C) pre_qr[n] = *reinterpret_cast<const u32x4*>(PQ + int64_t(dl_next[n]) * p.pqs_r + sch * 8);
+            pre_k[n] = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, kvoff[n], 0, 0);
+            pre_v[n] = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, vvoff[n], 0, 0);
+            if (HAS_C2P) pre_kr[n] = __builtin_amdgcn_raw_buffer_load_b128(pk_rsrc, dl_next[n] * pks_b + sch * 16, 0, 0);
+            if (HAS_P2C) pre_qr[n] = __builtin_amdgcn_raw_buffer_load_b128(pq_rsrc, dl_next[n] * pqs_b + sch * 16, 0, 0);
         }
     };
     auto fetch_delta = [&](int s) {      // delta of the 64 new window rows of key step s
@@ -218,7 +235,7 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const TdbKernelParams p)
     };
 
     // K fragments: A operand of S^T = K.Q^T, B operand of P'^T = Q_r'.K^T
-    bf16x8 kf[2][4];
+    bf16x8 kf[2][4], kf2[2][4];
     auto load_kf = [&](bf16x8 (&dst)[2][4]) {
 #pragma unroll
         for (int jt = 0; jt < 2; ++jt)
@@ -227,9 +244,10 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const TdbKernelParams p)
     };
     const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     const bool odd_wave = (w & 1) != 0;
-    // LDS reads of every A fragment the position products of one step need: c2p position tiles 0..2 of this wave's
-    // sub-window (fr[0..2]) and p2c position tiles w and 4 + w/2 of the workgroup window (fr[3], fr[4]).
-    auto load_pos_frags = [&](int off, bf16x8 (&fr)[5][4]) {
+    // LDS reads of the fragments the position products of one step need: c2p position tiles 0..2 of this wave's
+    // sub-window (fr[0..2]), p2c position tiles w and 4 + w/2 of the workgroup window (fr[3], fr[4]), and the key
+    // tile the latter is multiplied with (fr[5]).
+    auto load_pos_frags = [&](int off, bf16x8 (&fr)[6][4]) {
         auto ring = [&](int x) { const int t = x + off; return t >= WIN ? t - WIN : t; };
         if (HAS_C2P) {
 #pragma unroll
@@ -245,31 +263,32 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const TdbKernelParams p)
             for (int c = 0; c < 4; ++c) {
                 fr[3][c] = lds_frag(sm.qr, row3, 16 * c + 8 * hh);
                 fr[4][c] = lds_frag(sm.qr, row4, 16 * c + 8 * hh);
+                fr[5][c] = lds_frag(sm.k, 32 * (w & 1) + il, 16 * c + 8 * hh);   // keys of tile (w & 1): B operand of the third tile
             }
         }
     };
-    // Position products of one key step from fragments already in registers, into the scratch:
-    //   c2p  C'^T[r, i] = K_r'[r].Q_i over this wave's 96-position sub-window, stored as fp32 C'[i][r'];
-    //   p2c  P'^T[r, j] = Q_r'[r].K_j over the whole window (6 x 2 tiles): wave w takes position tile w against both
-    //        key tiles and tile (4 + w/2, w&1); stored as bf16 P'[j][r''].
-    auto pos_products = [&](const bf16x8 (&fr)[5][4], const bf16x8 (&kn)[2][4]) {
+    // Position products of one key step, tile by tile (each tile is a chain of 4 MFMAs over head_dim):
+    //   c2p  tiles 0..2: C'^T[r, i] = K_r'[r].Q_i over this wave's 96-position sub-window, stored as fp32 C'[i][r'];
+    //   p2c  tiles 3..5: P'^T[r, j] = Q_r'[r].K_j over the whole window (6 x 2 tiles): wave w takes position tile w
+    //        against both key tiles and tile (4 + w/2, w&1); stored as bf16 P'[j][r''].
+    auto put_c = [&](int rt, const f32x16& acc) {
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+            *reinterpret_cast<float4*>(&sm.c[w][il * CS + 32 * rt + 8 * a + 4 * hh]) =
+                float4{acc[4 * a], acc[4 * a + 1], acc[4 * a + 2], acc[4 * a + 3]};
+    };
+    auto put_p = [&](int rt, int jt, const f32x16& acc) {
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+            *reinterpret_cast<u32x2*>(&sm.p[(32 * jt + il) * PS + 32 * rt + 8 * a + 4 * hh]) =
+                pack4(acc[4 * a], acc[4 * a + 1], acc[4 * a + 2], acc[4 * a + 3]);
+    };
+    auto pos_products = [&](const bf16x8 (&fr)[6][4], const bf16x8 (&kn)[2][4]) {
         auto chain = [&](const bf16x8 (&a)[4], const bf16x8 (&bb)[4]) {
             f32x16 acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], bb[0], zero16, 0, 0, 0);
 #pragma unroll
             for (int c = 1; c < 4; ++c) acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[c], bb[c], acc, 0, 0, 0);
             return acc;
-        };
-        auto put_c = [&](int rt, const f32x16& acc) {
-#pragma unroll
-            for (int a = 0; a < 4; ++a)
-                *reinterpret_cast<float4*>(&sm.c[w][il * CS + 32 * rt + 8 * a + 4 * hh]) =
-                    float4{acc[4 * a], acc[4 * a + 1], acc[4 * a + 2], acc[4 * a + 3]};
-        };
-        auto put_p = [&](int rt, int jt, const f32x16& acc) {
-#pragma unroll
-            for (int a = 0; a < 4; ++a)
-                *reinterpret_cast<u32x2*>(&sm.p[(32 * jt + il) * PS + 32 * rt + 8 * a + 4 * hh]) =
-                    pack4(acc[4 * a], acc[4 * a + 1], acc[4 * a + 2], acc[4 * a + 3]);
         };
         if (HAS_C2P) {
             const f32x16 a0 = chain(fr[0], qb);
@@ -280,19 +299,10 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const TdbKernelParams p)
             put_c(2, a2);
         }
         if (HAS_P2C) {
-            bf16x8 kx[4];                 // key tile (w & 1), chosen without indexing registers
-#pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                const u32x4 x0 = __builtin_bit_cast(u32x4, kn[0][c]), x1 = __builtin_bit_cast(u32x4, kn[1][c]);
-                u32x4 r;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) r[e] = odd_wave ? x1[e] : x0[e];
-                kx[c] = __builtin_bit_cast(bf16x8, r);
-            }
             const f32x16 a0 = chain(fr[3], kn[0]);
             const f32x16 a1 = chain(fr[3], kn[1]);
             put_p(w, 0, a0);
-            const f32x16 a2 = chain(fr[4], kx);
+            const f32x16 a2 = chain(fr[4], fr[5]);
             put_p(w, 1, a1);
             put_p(4 + (w >> 1), w & 1, a2);
         }
@@ -322,20 +332,47 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const TdbKernelParams p)
     fetch_delta(2);
     load_kf(kf);
     {
-        bf16x8 fr[5][4];
+        bf16x8 fr[6][4];
         load_pos_frags(0, fr);
         pos_products(fr, kf);
     }
 
     TDB_T0();
+    // Probabilities (B operand of P.V, as packed bf16 pairs) and V^T fragments of the previous step: its P.V
+    // product is issued at the start of the next step's half A, under the scratch reads.
+    uint32_t pbw[2][2][4];                // [key tile][16-key chunk][dword]
+    bf16x8 vf[2][2][2];                   // [key tile][16-key chunk][dim tile]
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int b2 = 0; b2 < 2; ++b2) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) pbw[a][b2][e] = 0u;
+#pragma unroll
+            for (int d2 = 0; d2 < 2; ++d2) vf[a][b2][d2] = __builtin_bit_cast(bf16x8, u32x4{0, 0, 0, 0});
+        }
+    auto pv_product = [&]() {             // O^T += V^T.P^T
+#pragma unroll
+        for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+            for (int c = 0; c < 2; ++c) {
+                const u32x4 pw = {pbw[jt][c][0], pbw[jt][c][1], pbw[jt][c][2], pbw[jt][c][3]};
+#pragma unroll
+                for (int dt = 0; dt < 2; ++dt)
+                    o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[jt][c][dt], __builtin_bit_cast(bf16x8, pw), o_acc[dt], 0, 0, 0);
+            }
+    };
+
     // One key step.  MASKED: the step reaches past the end of the sequence (only the last step can).
-    auto key_step = [&](int s, int off, int off_next, auto masked_tag) {
+    auto key_step = [&](int s, int off_next, const bf16x8 (&kf)[2][4], bf16x8 (&kn)[2][4], auto masked_tag) {
         constexpr bool MASKED = decltype(masked_tag)::value;
         __syncthreads();                  // scratch of step s complete; every wave holds its K fragments of step s
         TDB_TICK(0);
 
-        // ---- half A: position terms of step s out of the scratch.  Element (jj, i) of the score tile takes
-        //      C'[i][i-jj+63] (fp32, straight into the accumulator) and P'[jj][32w+i-jj+63] (bf16) ----------------
+        // ---- half A: P.V of the previous step on the matrix cores while the position terms of step s come out of
+        //      the scratch.  Element (jj, i) of the score tile takes C'[i][i-jj+63] (fp32, straight into the
+        //      accumulator) and P'[jj][32w+i-jj+63] (bf16) -------------------------------------------------------
+        pv_product();
         f32x16 s_acc[2];
         if (HAS_C2P) {
             // float index of element e of key tile jt:  il*CS + il + 63 - 4*hh - jc,  jc = 32*jt + 8*(e>>2) + (e&3) <= 59
@@ -374,15 +411,14 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const TdbKernelParams p)
         __syncthreads();                  // scratch is free again; the staged tiles are visible
         TDB_TICK(2);
 
-        // ---- half B (one basic block, so that matrix and vector work can be interleaved) ------------------------
+        // ---- half B: one basic block, hand-interleaved: S^T(s) = K.Q^T on top of the position terms, then the
+        //      24 position MFMAs of step s+1 with the softmax of step s between them -----------------------------
         fetch(s + 2, s + 1);
         fetch_delta(s + 3);
-        bf16x8 kn[2][4], fr[5][4];
+        bf16x8 fr[6][4];
         load_kf(kn);                      // K fragments of step s+1
         load_pos_frags(off_next, fr);
-        // V^T fragments through the transposing LDS read: lane provides the address of 4 dims of one key
-        bf16x8 vf[2][2][2];               // [key tile][16-key chunk][dim tile]
-        {
+        {   // V^T fragments through the transposing LDS read: the lane provides the address of 4 dims of one key
             const int g = l >> 4, ll = l & 15;
             const uint16_t* vbase = &sm.v[((ll >> 2) + 4 * (g >> 1)) * RS + 16 * (g & 1) + 4 * (ll & 3)];
 #pragma unroll
@@ -402,8 +438,16 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const TdbKernelParams p)
         for (int c = 0; c < 4; ++c)
 #pragma unroll
             for (int jt = 0; jt < 2; ++jt) s_acc[jt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[jt][c], qb[c], s_acc[jt], 0, 0, 0);
-        pos_products(fr, kn);             // of step s+1 (harmless left-over work in the last step)
-        TDB_TICK(3);
+        __builtin_amdgcn_sched_barrier(0);
+
+        // position tile 0 goes to the matrix cores before the first instruction that needs the scores
+        f32x16 t0 = zero16, t1 = zero16, t2 = zero16, t3 = zero16, t4 = zero16, t5 = zero16;
+#define TDB_MF(acc, a, b) acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0)
+        if (HAS_C2P) {
+            TDB_MF(t0, fr[0][0], qb[0]); TDB_MF(t0, fr[0][1], qb[1]); TDB_MF(t0, fr[0][2], qb[2]); TDB_MF(t0, fr[0][3], qb[3]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+
         if (MASKED) {
 #pragma unroll
             for (int jt = 0; jt < 2; ++jt)
@@ -420,54 +464,94 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const TdbKernelParams p)
 #pragma unroll
             for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s_acc[jt][e]);
         mx = fmaxf(mx, __shfl_xor(mx, 32));
+        // The running maximum is only raised (and the accumulators rescaled) when some row of the wave exceeds it
+        // by more than 2^8; until then probabilities of this step may be as large as 256, which bf16 and the fp32
+        // sums carry exactly as well.  (First step: m_run = -inf always triggers, alpha = 0.)
         const float m_new = fmaxf(m_run, mx);          // finite: key 64s < len is never masked
-        const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * c_exp);
-        const float mc = m_new * c_exp;
-        m_run = m_new;
+        if (__builtin_amdgcn_ballot_w64((m_new - m_run) * c_exp > 8.f) != 0) {
+            const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * c_exp);
+            l_run *= alpha;
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) o_acc[t][e] *= alpha;
+            m_run = m_new;
+        }
+        const float mc = m_run * c_exp;
         float psum = 0.f;
-        bf16x8 pb[2][2];   // B operand of P.V: [key tile][16-key chunk]
+        // chunk g: 4 probabilities
+        auto sm_chunk = [&](auto gc) {
+            constexpr int g = decltype(gc)::value, jt = g >> 2, e0 = 4 * (g & 3);
+            float pe[4];
 #pragma unroll
-        for (int jt = 0; jt < 2; ++jt)
-#pragma unroll
-            for (int c = 0; c < 2; ++c) {
-                float pe[8];
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    pe[e] = __builtin_amdgcn_exp2f(fmaf(s_acc[jt][8 * c + e], c_exp, -mc));
-                    psum += pe[e];
-                }
-#pragma unroll
-                for (int e = 0; e < 8; ++e) pb[jt][c][e] = (__bf16)pe[e];
-            }
-        l_run = l_run * alpha + psum;
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) o_acc[t][e] *= alpha;
-        TDB_TICK(4);
-        // O^T += V^T.P^T
-#pragma unroll
-        for (int jt = 0; jt < 2; ++jt)
-#pragma unroll
-            for (int c = 0; c < 2; ++c)
-#pragma unroll
-                for (int dt = 0; dt < 2; ++dt)
-                    o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[jt][c][dt], pb[jt][c], o_acc[dt], 0, 0, 0);
-#pragma unroll
-        for (int jt = 0; jt < 2; ++jt)
-#pragma unroll
-            for (int c = 0; c < 4; ++c) kf[jt][c] = kn[jt][c];
-        TDB_TICK(5);
+            for (int e = 0; e < 4; ++e) pe[e] = __builtin_amdgcn_exp2f(fmaf(s_acc[jt][e0 + e], c_exp, -mc));
+            const bf16x2 lo = {(__bf16)pe[0], (__bf16)pe[1]}, hi = {(__bf16)pe[2], (__bf16)pe[3]};
+            psum = __builtin_amdgcn_fdot2_f32_bf16(lo, ones, psum, false);     // sum of what the MFMA will see
+            psum = __builtin_amdgcn_fdot2_f32_bf16(hi, ones, psum, false);
+            pbw[jt][(g & 3) >> 1][2 * (g & 1)] = __builtin_bit_cast(uint32_t, lo);
+            pbw[jt][(g & 3) >> 1][2 * (g & 1) + 1] = __builtin_bit_cast(uint32_t, hi);
+        };
+        // g0
+        if (HAS_C2P) { TDB_MF(t1, fr[1][0], qb[0]); TDB_MF(t1, fr[1][1], qb[1]); TDB_MF(t1, fr[1][2], qb[2]); }
+        sm_chunk(std::integral_constant<int, 0>{});
+        if (HAS_C2P) put_c(0, t0);
+        __builtin_amdgcn_sched_barrier(0);
+        // g1
+        if (HAS_C2P) { TDB_MF(t1, fr[1][3], qb[3]); TDB_MF(t2, fr[2][0], qb[0]); }
+        sm_chunk(std::integral_constant<int, 1>{});
+        __builtin_amdgcn_sched_barrier(0);
+        // g2
+        if (HAS_C2P) { TDB_MF(t2, fr[2][1], qb[1]); TDB_MF(t2, fr[2][2], qb[2]); TDB_MF(t2, fr[2][3], qb[3]); }
+        sm_chunk(std::integral_constant<int, 2>{});
+        __builtin_amdgcn_sched_barrier(0);
+        // g3
+        if (HAS_P2C) { TDB_MF(t3, fr[3][0], kn[0][0]); TDB_MF(t3, fr[3][1], kn[0][1]); }
+        sm_chunk(std::integral_constant<int, 3>{});
+        if (HAS_C2P) put_c(1, t1);
+        __builtin_amdgcn_sched_barrier(0);
+        // g4
+        if (HAS_P2C) { TDB_MF(t3, fr[3][2], kn[0][2]); TDB_MF(t3, fr[3][3], kn[0][3]); TDB_MF(t4, fr[3][0], kn[1][0]); }
+        sm_chunk(std::integral_constant<int, 4>{});
+        if (HAS_C2P) put_c(2, t2);
+        __builtin_amdgcn_sched_barrier(0);
+        // g5
+        if (HAS_P2C) { TDB_MF(t4, fr[3][1], kn[1][1]); TDB_MF(t4, fr[3][2], kn[1][2]); }
+        sm_chunk(std::integral_constant<int, 5>{});
+        __builtin_amdgcn_sched_barrier(0);
+        // g6
+        if (HAS_P2C) { TDB_MF(t4, fr[3][3], kn[1][3]); TDB_MF(t5, fr[4][0], fr[5][0]); TDB_MF(t5, fr[4][1], fr[5][1]); }
+        sm_chunk(std::integral_constant<int, 6>{});
+        if (HAS_P2C) put_p(w, 0, t3);
+        __builtin_amdgcn_sched_barrier(0);
+        // g7
+        if (HAS_P2C) { TDB_MF(t5, fr[4][2], fr[5][2]); TDB_MF(t5, fr[4][3], fr[5][3]); }
+        sm_chunk(std::integral_constant<int, 7>{});
+        __builtin_amdgcn_sched_barrier(0);
+#undef TDB_MF
+        l_run += psum;
+        if (HAS_P2C) {
+            put_p(w, 1, t4);
+            put_p(4 + (w >> 1), w & 1, t5);
+        }
+        TDB_TICK(3);
     };
 
+    // steps run in pairs so that the two sets of K fragment registers just swap roles
     int off = 0;                          // ring slot of window row 0 of the current step
+    auto next_off = [&]() { off = off >= BN ? off - BN : off + WIN - BN; return off; };
     const int nfull = len / BN;           // steps that need no key mask
-    for (int s = 0; s < nfull; ++s) {
-        const int off_next = off >= BN ? off - BN : off + WIN - BN;
-        key_step(s, off, off_next, std::false_type{});
-        off = off_next;
+    int s = 0;
+    for (; s + 1 < nfull; s += 2) {
+        key_step(s, next_off(), kf, kf2, std::false_type{});
+        key_step(s + 1, next_off(), kf2, kf, std::false_type{});
     }
-    if (nfull < nsteps) key_step(nfull, off, off >= BN ? off - BN : off + WIN - BN, std::true_type{});
+    if (s < nfull) {
+        key_step(s, next_off(), kf, kf2, std::false_type{});
+        if (nfull < nsteps) key_step(nfull, next_off(), kf2, kf, std::true_type{});
+    } else if (nfull < nsteps) {
+        key_step(nfull, next_off(), kf, kf2, std::true_type{});
+    }
+    pv_product();                         // of the last step
 
     // ---- epilogue: normalise and store O[i][d]; lane holds d = 32*dt + 8*a + 4*hh + 0..3 of query row il ------
     const float l_tot = l_run + __shfl_xor(l_run, 32);
