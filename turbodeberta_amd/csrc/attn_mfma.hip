@@ -1,20 +1,25 @@
 // Matrix-core disentangled-attention forward for bf16, head_dim 64 (gfx950, wave64, MFMA 32x32x16).
 //
-// One workgroup = 4 waves = one tile of 128 query rows of one (sequence, head); each wave owns 32
-// query rows and walks the keys 64 at a time with a streaming softmax.  Scores are kept
-// transposed (S^T = K.Q^T) so that a lane owns ONE query row: row max / row sum are in-lane
-// reductions plus one exchange between the two half-waves, and the S^T accumulator registers are
-// already the B operand of the P.V product (O^T += V^T.P^T), so probabilities never touch LDS.
+// One workgroup = one tile of 128 query rows of one (sequence, head), walked over the keys 64 at a
+// time.  It has 8 waves in two roles, paired on the SIMDs so that their matrix and vector work
+// interleave:
+//   * 4 "score" waves, 32 query rows each: S^T = K.Q^T on top of the position terms, streaming
+//     softmax, O^T += V^T.P^T.  Scores are kept transposed so that a lane owns ONE query row: row
+//     max / row sum are in-lane reductions plus one exchange between the half-waves, and the S^T
+//     accumulator registers are already the B operand of the P.V product, so probabilities never
+//     touch LDS.
+//   * 4 "position" waves: they stage K, V and the relative-position rows from global memory into
+//     LDS and compute, one key step ahead, the position products on the matrix cores.
 //
-// Position terms, per key step (j0 .. j0+63), in "position space": the workgroup needs relative
-// positions r = i - j in a window of 128+64-1 values.  Rows K_r[delta(r)] and Q_r[delta(r)] of the
-// per-head tables are staged in LDS for that window (delta from the host-built table, so log
+// Position terms, per key step (keys j0 .. j0+63), in "position space": the workgroup needs
+// relative positions r = i - j in a window of 128+64-1 values.  Rows K_r[delta(r)] and Q_r[delta(r)]
+// of the per-head tables are staged in LDS for that window (delta from the host-built table, so log
 // bucketing, saturation beyond max_relative_positions and the un-bucketed case are one code path
 // with bit-exact indices).  Then
-//   c2p:  C'^T[r, i] = K_r'[r] . Q_i      per wave, over its own 96-position sub-window,
+//   c2p:  C'^T[r, i] = K_r'[r] . Q_i      per 32-query block, over its own 96-position sub-window,
 //   p2c:  P'^T[r, j] = Q_r'[r] . K_j      once per workgroup,
-// both on MFMA, written to LDS (c2p as fp32, p2c as bf16) and read back skewed: score (i, j) takes C'[i][i-j] and
-// P'[j][i-j].  Score position (i, j) therefore gets Q_i.K_r[delta(i-j)] + K_j.Q_r[delta(i-j)], the
+// both on MFMA, written to LDS (c2p as fp32, p2c as bf16) and read back skewed by the score waves:
+// score (i, j) takes C'[i][i-j] and P'[j][i-j], i.e. Q_i.K_r[delta(i-j)] + K_j.Q_r[delta(i-j)], the
 // Hugging Face eager definition (modeling_deberta_v2.py:317-324, :337-343).
 #include <type_traits>
 #include <utility>
@@ -24,10 +29,10 @@
 namespace {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
-typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(4))) short s16x4;
+typedef __attribute__((ext_vector_type(8))) short s16x8;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 
@@ -36,7 +41,7 @@ typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 // Phase timing for development builds (-DTDB_TIMING): one wave accumulates cycle counts per phase.
 #ifdef TDB_TIMING
 __device__ long long tdb_timing[16];
-#define TDB_T0() long long tdb_t = clock64(); const bool tdb_on = blockIdx.x == 7 && blockIdx.y == 3 && threadIdx.x == 64
+#define TDB_T0(t) long long tdb_t = clock64(); const bool tdb_on = blockIdx.x == 7 && blockIdx.y == 3 && threadIdx.x == (t)
 #define TDB_TICK(k)                                        \
     do {                                                   \
         const long long n_ = clock64();                    \
@@ -44,17 +49,19 @@ __device__ long long tdb_timing[16];
         tdb_t = n_;                                        \
     } while (0)
 #else
-#define TDB_T0() do {} while (0)
+#define TDB_T0(t) do {} while (0)
 #define TDB_TICK(k) do {} while (0)
 #endif
 
 constexpr int BM = TDB_MFMA_TILE;   // query rows per workgroup
 constexpr int BN = 64;              // keys per step
 constexpr int D = 64;
+constexpr int NTHREADS = 512;       // 4 score waves + 4 position waves
 constexpr int WIN = BM + BN;        // ring of staged window rows (one more than the 191 positions in use)
 constexpr int RS = 72;              // LDS row stride (elements) of 64-wide bf16 rows: 144 B, conflict-free b128
-constexpr int CS = 100;             // row stride (floats) of the per-wave c2p scratch [32][96 used]
-constexpr int PS = 196;             // row stride of the p2c scratch           [64][192 used]
+constexpr int CS = 100;             // row stride (floats) of the per-block c2p scratch [32][96 used]
+constexpr int PS = 196;             // row stride of the p2c scratch                   [64][192 used]
+constexpr int RSRC_FLAGS = 0x00020000;   // raw buffer resource, 32-bit data format
 
 struct Smem {
     uint16_t k[BN * RS];
@@ -118,12 +125,15 @@ __device__ __forceinline__ uint32_t lds_addr(const void* p) {
 }
 
 template <bool HAS_C2P, bool HAS_P2C>
-__global__ __launch_bounds__(256) void attn_mfma_kernel(const TdbKernelParams p) {
+__global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelParams p) {
     extern __shared__ __attribute__((aligned(16))) char smem_raw[];
     Smem& sm = *reinterpret_cast<Smem*>(smem_raw);
+    constexpr bool HAS_POS = HAS_C2P || HAS_P2C;
 
     const int tid = threadIdx.x;
-    const int w = tid >> 6, l = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const bool score_role = wave < 4;     // waves 0..3 score, 4..7 position; wave w and w+4 share query block w
+    const int w = wave & 3, l = tid & 63;
     const int il = l & 31, hh = l >> 5;
     const int head = blockIdx.y;
 
@@ -138,15 +148,17 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const TdbKernelParams p)
     const int rows_here = min(BM, (p.varlen ? len : p.L) - row0);   // rows of this tile that exist in memory
 
     if (row0 >= len) {   // only padded query rows (fixed layout): zeros
-        for (int idx = tid; idx < rows_here * (D / 8); idx += 256)
+        for (int idx = tid; idx < rows_here * (D / 8); idx += NTHREADS)
             *reinterpret_cast<u32x4*>(O + int64_t(row0 + (idx >> 3)) * p.os_l + (idx & 7) * 8) = u32x4{0, 0, 0, 0};
         return;
     }
 
     const uint16_t* PK = HAS_C2P ? static_cast<const uint16_t*>(p.pk) + int64_t(head) * p.pks_h : nullptr;
     const uint16_t* PQ = HAS_P2C ? static_cast<const uint16_t*>(p.pq) + int64_t(head) * p.pqs_h : nullptr;
+    const int lut_max = 2 * p.lut_half;
+    auto delta_of = [&](int r) { return p.lut[min(max(r + p.lut_half, 0), lut_max)]; };
 
-    // B operand of every product against this wave's queries: Q^T, k = d.
+    // Q^T fragments of query block w: B operand of S^T = K.Q^T (score wave) and of C'^T = K_r'.Q^T (position wave)
     const int qi = row0 + 32 * w + il;
     bf16x8 qb[4];
 #pragma unroll
@@ -156,17 +168,6 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const TdbKernelParams p)
         qb[c] = __builtin_bit_cast(bf16x8, t);
     }
 
-    f32x16 o_acc[2];
-#pragma unroll
-    for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) o_acc[t][e] = 0.f;
-    float m_run = -INFINITY, l_run = 0.f;
-    const float c_exp = p.scale * 1.4426950408889634f;   // softmax in base 2
-
-    const int lut_max = 2 * p.lut_half;
-    const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
-
     // ---- pipeline ----------------------------------------------------------------------------------------------
     // Key step s covers keys 64s .. 64s+63 and needs relative positions B_s .. B_s+190, B_s = row0 - 64s - 63.
     // The rows K_r[delta(r)] / Q_r[delta(r)] of that window live in a 192-row ring: going to the next step the
@@ -174,205 +175,209 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const TdbKernelParams p)
     // of the previous step.  Window row x of step s sits in ring slot (x + off_s) mod 192, off_s = (128*s) mod 192.
     //
     // Each step has two halves separated by workgroup barriers:
-    //   A  read this step's position terms out of the C'/P' scratch (into the score accumulators) and hand the
-    //      register-prefetched global data to LDS: keys of step s+1, values of step s, 64 window rows of step s+1;
-    //   B  matrix work: S^T(s) = K.Q^T on top of the position terms, then the position products C', P' of step
-    //      s+1 into the now free scratch, softmax(s) on the vector ALUs, P.V(s); global fetches for half A of the
-    //      next step are issued at the start of B.
-    // The K fragments of step s+1 are read from LDS in half B (for P'(s+1)) and stay in registers for S^T(s+1).
-    constexpr bool HAS_POS = HAS_C2P || HAS_P2C;
+    //   A  score waves read this step's position terms out of the C'/P' scratch into their score accumulators;
+    //      position waves hand their register-prefetched global data to LDS: keys of step s+1, values of step s,
+    //      64 window rows of step s+1;
+    //   B  score waves: S^T(s), softmax(s), P.V(s), and they pick up the K fragments of step s+1;
+    //      position waves: global fetches for the next half A, then the position products C', P' of step s+1 into
+    //      the now free scratch.
     const int nsteps = (len + BN - 1) / BN;
-    const int srow = tid >> 3, sch = tid & 7;              // this thread stages rows srow, srow+32 (chunk sch)
-    auto delta_of = [&](int r) { return p.lut[min(max(r + p.lut_half, 0), lut_max)]; };
+    const int nfull = len / BN;           // steps that need no key mask
+    int off = 0;                          // ring slot of window row 0 of the current step
+    auto next_off = [&]() { off = off >= BN ? off - BN : off + WIN - BN; return off; };
+    const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
-    u32x4 pre_k[2], pre_v[2], pre_kr[2], pre_qr[2];
-    int dl_next[2] = {0, 0};
-    // global -> registers through buffer loads: key rows of step sk, value rows of step sv, the 64 new window rows
-    // whose delta is in dl_next.  The buffer of a step starts at its first row and ends with the last row of the
-    // sequence, so rows past the end come back as zeros (hardware range check) with no lane predicated off, and the
-    // only per-load address arithmetic left is scalar.
-    const int ks_b = int(p.ks_l) * 2, vs_b = int(p.vs_l) * 2, pks_b = int(p.pks_r) * 2, pqs_b = int(p.pqs_r) * 2;
-    int kvoff[2], vvoff[2];               // byte offsets of this thread's two rows inside a step's buffer
-#pragma unroll
-    for (int n = 0; n < 2; ++n) {
-        kvoff[n] = (srow + 32 * n) * ks_b + sch * 16;
-        vvoff[n] = (srow + 32 * n) * vs_b + sch * 16;
-    }
-    constexpr int RSRC_FLAGS = 0x00020000;   // raw buffer, 32-bit data format
-    const __amdgpu_buffer_rsrc_t pk_rsrc =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(HAS_C2P ? PK : K), 0, HAS_C2P ? (2 * p.span - 1) * pks_b + 128 : 0, RSRC_FLAGS);
-    const __amdgpu_buffer_rsrc_t pq_rsrc =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(HAS_P2C ? PQ : K), 0, HAS_P2C ? (2 * p.span - 1) * pqs_b + 128 : 0, RSRC_FLAGS);
-    auto fetch = [&](int sk, int sv) {
-        const int kleft = len - BN * sk, vleft = len - BN * sv;      // rows of the sequence from the step's first row on
-        const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-            const_cast<uint16_t*>(K) + int64_t(BN * sk) * p.ks_l, 0, kleft > 0 ? (kleft - 1) * ks_b + 128 : 0, RSRC_FLAGS);
-        const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-            const_cast<uint16_t*>(V) + int64_t(BN * sv) * p.vs_l, 0, vleft > 0 ? (vleft - 1) * vs_b + 128 : 0, RSRC_FLAGS);
-#pragma unroll
-        for (int n = 0; n < 2; ++n) {
-            pre_k[n] = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, kvoff[n], 0, 0);
-            pre_v[n] = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, vvoff[n], 0, 0);
-            if (HAS_C2P) pre_kr[n] = __builtin_amdgcn_raw_buffer_load_b128(pk_rsrc, dl_next[n] * pks_b + sch * 16, 0, 0);
-            if (HAS_P2C) pre_qr[n] = __builtin_amdgcn_raw_buffer_load_b128(pq_rsrc, dl_next[n] * pqs_b + sch * 16, 0, 0);
-        }
-    };
-    auto fetch_delta = [&](int s) {      // delta of the 64 new window rows of key step s
+    // prologue, all 512 threads: keys and whole window of step 0 to LDS
+    {
+        const int row = tid >> 3, ch = tid & 7;              // rows 0..63
+        *reinterpret_cast<u32x4*>(&sm.k[row * RS + ch * 8]) =
+            *reinterpret_cast<const u32x4*>(K + int64_t(min(row, len - 1)) * p.ks_l + ch * 8);
         if (HAS_POS) {
 #pragma unroll
-            for (int n = 0; n < 2; ++n) dl_next[n] = delta_of(row0 - BN * s - (BN - 1) + srow + 32 * n);
+            for (int n = 0; n < WIN / 64; ++n) {
+                const int x = row + 64 * n;
+                const int dl = delta_of(row0 - (BN - 1) + x);
+                if (HAS_C2P)
+                    *reinterpret_cast<u32x4*>(&sm.kr[x * RS + ch * 8]) = *reinterpret_cast<const u32x4*>(PK + int64_t(dl) * p.pks_r + ch * 8);
+                if (HAS_P2C)
+                    *reinterpret_cast<u32x4*>(&sm.qr[x * RS + ch * 8]) = *reinterpret_cast<const u32x4*>(PQ + int64_t(dl) * p.pqs_r + ch * 8);
+            }
         }
-    };
-    auto store = [&](int off) {          // registers -> LDS
+    }
+    __syncthreads();
+
+    if (!score_role) {
+        // ================================================= position waves ==========================================
+        const int stid = tid - 256;
+        TDB_T0(320);
+        const int srow = stid >> 3, sch = stid & 7;          // this thread stages rows srow, srow+32 (chunk sch)
+        // global -> registers through buffer loads.  The buffer of a step starts at its first row and ends with the
+        // last row of the sequence, so rows past the end come back as zeros (hardware range check) with no lane
+        // predicated off, and the per-load address arithmetic is scalar.
+        const int ks_b = int(p.ks_l) * 2, vs_b = int(p.vs_l) * 2, pks_b = int(p.pks_r) * 2, pqs_b = int(p.pqs_r) * 2;
+        int kvoff[2], vvoff[2];
 #pragma unroll
         for (int n = 0; n < 2; ++n) {
-            const int r = srow + 32 * n;
-            *reinterpret_cast<u32x4*>(&sm.k[r * RS + sch * 8]) = pre_k[n];
-            *reinterpret_cast<u32x4*>(&sm.v[r * RS + sch * 8]) = pre_v[n];
-            if (HAS_C2P) *reinterpret_cast<u32x4*>(&sm.kr[(off + r) * RS + sch * 8]) = pre_kr[n];
-            if (HAS_P2C) *reinterpret_cast<u32x4*>(&sm.qr[(off + r) * RS + sch * 8]) = pre_qr[n];
+            kvoff[n] = (srow + 32 * n) * ks_b + sch * 16;
+            vvoff[n] = (srow + 32 * n) * vs_b + sch * 16;
         }
-    };
+        const __amdgpu_buffer_rsrc_t pk_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<uint16_t*>(HAS_C2P ? PK : K), 0, HAS_C2P ? (2 * p.span - 1) * pks_b + 128 : 0, RSRC_FLAGS);
+        const __amdgpu_buffer_rsrc_t pq_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<uint16_t*>(HAS_P2C ? PQ : K), 0, HAS_P2C ? (2 * p.span - 1) * pqs_b + 128 : 0, RSRC_FLAGS);
+        u32x4 pre_k[2], pre_v[2], pre_kr[2], pre_qr[2];
+        int dl_next[2] = {0, 0};
+        auto fetch = [&](int sk, int sv) {     // key rows of step sk, value rows of step sv, new window rows (dl_next)
+            const int kleft = len - BN * sk, vleft = len - BN * sv;
+            const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+                const_cast<uint16_t*>(K) + int64_t(BN * sk) * p.ks_l, 0, kleft > 0 ? (kleft - 1) * ks_b + 128 : 0, RSRC_FLAGS);
+            const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+                const_cast<uint16_t*>(V) + int64_t(BN * sv) * p.vs_l, 0, vleft > 0 ? (vleft - 1) * vs_b + 128 : 0, RSRC_FLAGS);
+#pragma unroll
+            for (int n = 0; n < 2; ++n) {
+                pre_k[n] = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, kvoff[n], 0, 0);
+                pre_v[n] = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, vvoff[n], 0, 0);
+                if (HAS_C2P) pre_kr[n] = __builtin_amdgcn_raw_buffer_load_b128(pk_rsrc, dl_next[n] * pks_b + sch * 16, 0, 0);
+                if (HAS_P2C) pre_qr[n] = __builtin_amdgcn_raw_buffer_load_b128(pq_rsrc, dl_next[n] * pqs_b + sch * 16, 0, 0);
+            }
+        };
+        auto fetch_delta = [&](int s) {        // delta of the 64 new window rows of key step s
+            if (HAS_POS) {
+#pragma unroll
+                for (int n = 0; n < 2; ++n) dl_next[n] = delta_of(row0 - BN * s - (BN - 1) + srow + 32 * n);
+            }
+        };
+        auto store = [&](int o) {              // registers -> LDS
+#pragma unroll
+            for (int n = 0; n < 2; ++n) {
+                const int r = srow + 32 * n;
+                *reinterpret_cast<u32x4*>(&sm.k[r * RS + sch * 8]) = pre_k[n];
+                *reinterpret_cast<u32x4*>(&sm.v[r * RS + sch * 8]) = pre_v[n];
+                if (HAS_C2P) *reinterpret_cast<u32x4*>(&sm.kr[(o + r) * RS + sch * 8]) = pre_kr[n];
+                if (HAS_P2C) *reinterpret_cast<u32x4*>(&sm.qr[(o + r) * RS + sch * 8]) = pre_qr[n];
+            }
+        };
+        // Position products of one key step from the ring at offset o and the keys in sm.k, into the scratch:
+        //   c2p  C'^T[r, i] = K_r'[r].Q_i over the 96-position sub-window of query block w, stored as fp32 C'[i][r'];
+        //   p2c  P'^T[r, j] = Q_r'[r].K_j over the whole window (6 x 2 tiles): wave w takes position tile w against
+        //        both key tiles and tile (4 + w/2, w&1); stored as bf16 P'[j][r''].
+        auto pos_products = [&](int o) {
+            auto ring = [&](int x) { const int t = x + o; return t >= WIN ? t - WIN : t; };
+            auto chain = [&](const bf16x8 (&a)[4], const bf16x8 (&bb)[4]) {
+                f32x16 acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], bb[0], zero16, 0, 0, 0);
+#pragma unroll
+                for (int c = 1; c < 4; ++c) acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[c], bb[c], acc, 0, 0, 0);
+                return acc;
+            };
+            auto put_c = [&](int rt, const f32x16& acc) {
+#pragma unroll
+                for (int a = 0; a < 4; ++a)
+                    *reinterpret_cast<float4*>(&sm.c[w][il * CS + 32 * rt + 8 * a + 4 * hh]) =
+                        float4{acc[4 * a], acc[4 * a + 1], acc[4 * a + 2], acc[4 * a + 3]};
+            };
+            auto put_p = [&](int rt, int jt, const f32x16& acc) {
+#pragma unroll
+                for (int a = 0; a < 4; ++a)
+                    *reinterpret_cast<u32x2*>(&sm.p[(32 * jt + il) * PS + 32 * rt + 8 * a + 4 * hh]) =
+                        pack4(acc[4 * a], acc[4 * a + 1], acc[4 * a + 2], acc[4 * a + 3]);
+            };
+            bf16x8 fr[3][4], fq[2][4], kb[3][4];
+            if (HAS_C2P) {
+#pragma unroll
+                for (int rt = 0; rt < 3; ++rt) {
+                    const int row = ring(32 * w + 32 * rt + il);
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) fr[rt][c] = lds_frag(sm.kr, row, 16 * c + 8 * hh);
+                }
+            }
+            if (HAS_P2C) {
+                const int row3 = ring(32 * w + il), row4 = ring(32 * (4 + (w >> 1)) + il);
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    fq[0][c] = lds_frag(sm.qr, row3, 16 * c + 8 * hh);
+                    fq[1][c] = lds_frag(sm.qr, row4, 16 * c + 8 * hh);
+                    kb[0][c] = lds_frag(sm.k, il, 16 * c + 8 * hh);
+                    kb[1][c] = lds_frag(sm.k, 32 + il, 16 * c + 8 * hh);
+                }
+            }
+            // every fragment read is in flight before the first MFMA waits for one
+            __builtin_amdgcn_sched_barrier(0);
+            TDB_TICK(8);
+            if (HAS_P2C) {
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {   // key tile (w & 1), chosen without indexing registers
+                    const u32x4 x0 = __builtin_bit_cast(u32x4, kb[0][c]), x1 = __builtin_bit_cast(u32x4, kb[1][c]);
+                    u32x4 r;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) r[e] = (w & 1) ? x1[e] : x0[e];
+                    kb[2][c] = __builtin_bit_cast(bf16x8, r);
+                }
+            }
+            if (HAS_C2P) {
+                const f32x16 a0 = chain(fr[0], qb);
+                const f32x16 a1 = chain(fr[1], qb);
+                put_c(0, a0);
+                const f32x16 a2 = chain(fr[2], qb);
+                put_c(1, a1);
+                put_c(2, a2);
+            }
+            TDB_TICK(9);
+            if (HAS_P2C) {
+                const f32x16 a0 = chain(fq[0], kb[0]);
+                const f32x16 a1 = chain(fq[0], kb[1]);
+                put_p(w, 0, a0);
+                const f32x16 a2 = chain(fq[1], kb[2]);
+                put_p(w, 1, a1);
+                put_p(4 + (w >> 1), w & 1, a2);
+            }
+        };
 
-    // K fragments: A operand of S^T = K.Q^T, B operand of P'^T = Q_r'.K^T
-    bf16x8 kf[2][4], kf2[2][4];
+        fetch_delta(1);
+        fetch(1, 0);
+        fetch_delta(2);
+        pos_products(0);
+        TDB_TICK(11);
+        for (int s = 0; s < nsteps; ++s) {
+            const int off_next = next_off();
+            __syncthreads();              // scratch of step s complete
+            TDB_TICK(4);
+            store(off_next);              // keys of step s+1, values of step s, new window rows of step s+1
+            TDB_TICK(5);
+            __syncthreads();              // scratch is free again; the staged tiles are visible
+            TDB_TICK(6);
+            fetch(s + 2, s + 1);
+            fetch_delta(s + 3);
+            TDB_TICK(7);
+            pos_products(off_next);       // of step s+1 (harmless left-over work in the last step)
+            TDB_TICK(10);
+        }
+        return;
+    }
+
+    // ===================================================== score waves ============================================
+    f32x16 o_acc[2] = {zero16, zero16};
+    float m_run = -INFINITY, l_run = 0.f;
+    const float c_exp = p.scale * 1.4426950408889634f;   // softmax in base 2
+    const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
+
+    bf16x8 kf[2][4], kf2[2][4];           // K fragments: A operand of S^T = K.Q^T; two sets that swap roles
     auto load_kf = [&](bf16x8 (&dst)[2][4]) {
 #pragma unroll
         for (int jt = 0; jt < 2; ++jt)
 #pragma unroll
             for (int c = 0; c < 4; ++c) dst[jt][c] = lds_frag(sm.k, 32 * jt + il, 16 * c + 8 * hh);
     };
-    const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    const bool odd_wave = (w & 1) != 0;
-    // LDS reads of the fragments the position products of one step need: c2p position tiles 0..2 of this wave's
-    // sub-window (fr[0..2]), p2c position tiles w and 4 + w/2 of the workgroup window (fr[3], fr[4]), and the key
-    // tile the latter is multiplied with (fr[5]).
-    auto load_pos_frags = [&](int off, bf16x8 (&fr)[6][4]) {
-        auto ring = [&](int x) { const int t = x + off; return t >= WIN ? t - WIN : t; };
-        if (HAS_C2P) {
-#pragma unroll
-            for (int rt = 0; rt < 3; ++rt) {
-                const int row = ring(32 * w + 32 * rt + il);
-#pragma unroll
-                for (int c = 0; c < 4; ++c) fr[rt][c] = lds_frag(sm.kr, row, 16 * c + 8 * hh);
-            }
-        }
-        if (HAS_P2C) {
-            const int row3 = ring(32 * w + il), row4 = ring(32 * (4 + (w >> 1)) + il);
-#pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                fr[3][c] = lds_frag(sm.qr, row3, 16 * c + 8 * hh);
-                fr[4][c] = lds_frag(sm.qr, row4, 16 * c + 8 * hh);
-                fr[5][c] = lds_frag(sm.k, 32 * (w & 1) + il, 16 * c + 8 * hh);   // keys of tile (w & 1): B operand of the third tile
-            }
-        }
-    };
-    // Position products of one key step, tile by tile (each tile is a chain of 4 MFMAs over head_dim):
-    //   c2p  tiles 0..2: C'^T[r, i] = K_r'[r].Q_i over this wave's 96-position sub-window, stored as fp32 C'[i][r'];
-    //   p2c  tiles 3..5: P'^T[r, j] = Q_r'[r].K_j over the whole window (6 x 2 tiles): wave w takes position tile w
-    //        against both key tiles and tile (4 + w/2, w&1); stored as bf16 P'[j][r''].
-    auto put_c = [&](int rt, const f32x16& acc) {
-#pragma unroll
-        for (int a = 0; a < 4; ++a)
-            *reinterpret_cast<float4*>(&sm.c[w][il * CS + 32 * rt + 8 * a + 4 * hh]) =
-                float4{acc[4 * a], acc[4 * a + 1], acc[4 * a + 2], acc[4 * a + 3]};
-    };
-    auto put_p = [&](int rt, int jt, const f32x16& acc) {
-#pragma unroll
-        for (int a = 0; a < 4; ++a)
-            *reinterpret_cast<u32x2*>(&sm.p[(32 * jt + il) * PS + 32 * rt + 8 * a + 4 * hh]) =
-                pack4(acc[4 * a], acc[4 * a + 1], acc[4 * a + 2], acc[4 * a + 3]);
-    };
-    auto pos_products = [&](const bf16x8 (&fr)[6][4], const bf16x8 (&kn)[2][4]) {
-        auto chain = [&](const bf16x8 (&a)[4], const bf16x8 (&bb)[4]) {
-            f32x16 acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], bb[0], zero16, 0, 0, 0);
-#pragma unroll
-            for (int c = 1; c < 4; ++c) acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[c], bb[c], acc, 0, 0, 0);
-            return acc;
-        };
-        if (HAS_C2P) {
-            const f32x16 a0 = chain(fr[0], qb);
-            const f32x16 a1 = chain(fr[1], qb);
-            put_c(0, a0);
-            const f32x16 a2 = chain(fr[2], qb);
-            put_c(1, a1);
-            put_c(2, a2);
-        }
-        if (HAS_P2C) {
-            const f32x16 a0 = chain(fr[3], kn[0]);
-            const f32x16 a1 = chain(fr[3], kn[1]);
-            put_p(w, 0, a0);
-            const f32x16 a2 = chain(fr[4], fr[5]);
-            put_p(w, 1, a1);
-            put_p(4 + (w >> 1), w & 1, a2);
-        }
-    };
-
-    // prologue: keys and whole window of step 0 to LDS, position products of step 0, prefetch for half A of step 0
-    if (HAS_POS) {
-#pragma unroll
-        for (int n = 0; n < WIN * 8 / 256; ++n) {
-            const int x = srow + 32 * n;
-            const int dl = delta_of(row0 - (BN - 1) + x);
-            if (HAS_C2P)
-                *reinterpret_cast<u32x4*>(&sm.kr[x * RS + sch * 8]) = *reinterpret_cast<const u32x4*>(PK + int64_t(dl) * p.pks_r + sch * 8);
-            if (HAS_P2C)
-                *reinterpret_cast<u32x4*>(&sm.qr[x * RS + sch * 8]) = *reinterpret_cast<const u32x4*>(PQ + int64_t(dl) * p.pqs_r + sch * 8);
-        }
-    }
-#pragma unroll
-    for (int n = 0; n < 2; ++n) {
-        const int r = srow + 32 * n;
-        *reinterpret_cast<u32x4*>(&sm.k[r * RS + sch * 8]) =
-            *reinterpret_cast<const u32x4*>(K + int64_t(min(r, len - 1)) * p.ks_l + sch * 8);
-    }
-    fetch_delta(1);
-    __syncthreads();
-    fetch(1, 0);
-    fetch_delta(2);
     load_kf(kf);
-    {
-        bf16x8 fr[6][4];
-        load_pos_frags(0, fr);
-        pos_products(fr, kf);
-    }
 
-    TDB_T0();
-    // Probabilities (B operand of P.V, as packed bf16 pairs) and V^T fragments of the previous step: its P.V
-    // product is issued at the start of the next step's half A, under the scratch reads.
-    uint32_t pbw[2][2][4];                // [key tile][16-key chunk][dword]
-    bf16x8 vf[2][2][2];                   // [key tile][16-key chunk][dim tile]
-#pragma unroll
-    for (int a = 0; a < 2; ++a)
-#pragma unroll
-        for (int b2 = 0; b2 < 2; ++b2) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e) pbw[a][b2][e] = 0u;
-#pragma unroll
-            for (int d2 = 0; d2 < 2; ++d2) vf[a][b2][d2] = __builtin_bit_cast(bf16x8, u32x4{0, 0, 0, 0});
-        }
-    auto pv_product = [&]() {             // O^T += V^T.P^T
-#pragma unroll
-        for (int jt = 0; jt < 2; ++jt)
-#pragma unroll
-            for (int c = 0; c < 2; ++c) {
-                const u32x4 pw = {pbw[jt][c][0], pbw[jt][c][1], pbw[jt][c][2], pbw[jt][c][3]};
-#pragma unroll
-                for (int dt = 0; dt < 2; ++dt)
-                    o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[jt][c][dt], __builtin_bit_cast(bf16x8, pw), o_acc[dt], 0, 0, 0);
-            }
-    };
-
+    TDB_T0(64);
     // One key step.  MASKED: the step reaches past the end of the sequence (only the last step can).
-    auto key_step = [&](int s, int off_next, const bf16x8 (&kf)[2][4], bf16x8 (&kn)[2][4], auto masked_tag) {
+    auto key_step = [&](int s, const bf16x8 (&kc)[2][4], bf16x8 (&kn)[2][4], auto masked_tag) {
         constexpr bool MASKED = decltype(masked_tag)::value;
-        __syncthreads();                  // scratch of step s complete; every wave holds its K fragments of step s
+        __syncthreads();                  // scratch of step s complete
         TDB_TICK(0);
 
-        // ---- half A: P.V of the previous step on the matrix cores while the position terms of step s come out of
-        //      the scratch.  Element (jj, i) of the score tile takes C'[i][i-jj+63] (fp32, straight into the
-        //      accumulator) and P'[jj][32w+i-jj+63] (bf16) -------------------------------------------------------
-        pv_product();
+        // ---- half A: position terms of step s out of the scratch.  Element (jj, i) of the score tile takes
+        //      C'[i][i-jj+63] (fp32, straight into the accumulator) and P'[jj][32w+i-jj+63] (bf16) ----------------
         f32x16 s_acc[2];
         if (HAS_C2P) {
             // float index of element e of key tile jt:  il*CS + il + 63 - 4*hh - jc,  jc = 32*jt + 8*(e>>2) + (e&3) <= 59
@@ -406,19 +411,19 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const TdbKernelParams p)
                 for (int e = 0; e < 16; ++e)   // bf16 pair (value, 0) . (1, 1) + acc
                     s_acc[jt][e] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, g[jt][e]), ones, s_acc[jt][e], false);
         }
-        store(off_next);                  // keys of step s+1, values of step s, new window rows of step s+1
         TDB_TICK(1);
-        __syncthreads();                  // scratch is free again; the staged tiles are visible
+        __syncthreads();                  // scratch is free again; keys of step s+1 and values of step s are staged
         TDB_TICK(2);
 
-        // ---- half B: one basic block, hand-interleaved: S^T(s) = K.Q^T on top of the position terms, then the
-        //      24 position MFMAs of step s+1 with the softmax of step s between them -----------------------------
-        fetch(s + 2, s + 1);
-        fetch_delta(s + 3);
-        bf16x8 fr[6][4];
+        // ---- half B ---------------------------------------------------------------------------------------------
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+#pragma unroll
+            for (int jt = 0; jt < 2; ++jt) s_acc[jt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kc[jt][c], qb[c], s_acc[jt], 0, 0, 0);
         load_kf(kn);                      // K fragments of step s+1
-        load_pos_frags(off_next, fr);
-        {   // V^T fragments through the transposing LDS read: the lane provides the address of 4 dims of one key
+        // V^T fragments through the transposing LDS read: the lane provides the address of 4 dims of one key
+        bf16x8 vf[2][2][2];               // [key tile][16-key chunk][dim tile]
+        {
             const int g = l >> 4, ll = l & 15;
             const uint16_t* vbase = &sm.v[((ll >> 2) + 4 * (g >> 1)) * RS + 16 * (g & 1) + 4 * (ll & 3)];
 #pragma unroll
@@ -430,24 +435,10 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const TdbKernelParams p)
                         const uint16_t* src = vbase + (32 * jt + 16 * c) * RS + 32 * dt;
                         const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(TDB_LDS(s16x4, src));
                         const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(TDB_LDS(s16x4, src + 8 * RS));
-                        const __attribute__((ext_vector_type(8))) short both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                        const s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
                         vf[jt][c][dt] = __builtin_bit_cast(bf16x8, both);
                     }
         }
-#pragma unroll
-        for (int c = 0; c < 4; ++c)
-#pragma unroll
-            for (int jt = 0; jt < 2; ++jt) s_acc[jt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[jt][c], qb[c], s_acc[jt], 0, 0, 0);
-        __builtin_amdgcn_sched_barrier(0);
-
-        // position tile 0 goes to the matrix cores before the first instruction that needs the scores
-        f32x16 t0 = zero16, t1 = zero16, t2 = zero16, t3 = zero16, t4 = zero16, t5 = zero16;
-#define TDB_MF(acc, a, b) acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0)
-        if (HAS_C2P) {
-            TDB_MF(t0, fr[0][0], qb[0]); TDB_MF(t0, fr[0][1], qb[1]); TDB_MF(t0, fr[0][2], qb[2]); TDB_MF(t0, fr[0][3], qb[3]);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-
         if (MASKED) {
 #pragma unroll
             for (int jt = 0; jt < 2; ++jt)
@@ -479,79 +470,41 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const TdbKernelParams p)
         }
         const float mc = m_run * c_exp;
         float psum = 0.f;
-        // chunk g: 4 probabilities
-        auto sm_chunk = [&](auto gc) {
-            constexpr int g = decltype(gc)::value, jt = g >> 2, e0 = 4 * (g & 3);
-            float pe[4];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) pe[e] = __builtin_amdgcn_exp2f(fmaf(s_acc[jt][e0 + e], c_exp, -mc));
-            const bf16x2 lo = {(__bf16)pe[0], (__bf16)pe[1]}, hi = {(__bf16)pe[2], (__bf16)pe[3]};
-            psum = __builtin_amdgcn_fdot2_f32_bf16(lo, ones, psum, false);     // sum of what the MFMA will see
-            psum = __builtin_amdgcn_fdot2_f32_bf16(hi, ones, psum, false);
-            pbw[jt][(g & 3) >> 1][2 * (g & 1)] = __builtin_bit_cast(uint32_t, lo);
-            pbw[jt][(g & 3) >> 1][2 * (g & 1) + 1] = __builtin_bit_cast(uint32_t, hi);
-        };
-        // g0
-        if (HAS_C2P) { TDB_MF(t1, fr[1][0], qb[0]); TDB_MF(t1, fr[1][1], qb[1]); TDB_MF(t1, fr[1][2], qb[2]); }
-        sm_chunk(std::integral_constant<int, 0>{});
-        if (HAS_C2P) put_c(0, t0);
-        __builtin_amdgcn_sched_barrier(0);
-        // g1
-        if (HAS_C2P) { TDB_MF(t1, fr[1][3], qb[3]); TDB_MF(t2, fr[2][0], qb[0]); }
-        sm_chunk(std::integral_constant<int, 1>{});
-        __builtin_amdgcn_sched_barrier(0);
-        // g2
-        if (HAS_C2P) { TDB_MF(t2, fr[2][1], qb[1]); TDB_MF(t2, fr[2][2], qb[2]); TDB_MF(t2, fr[2][3], qb[3]); }
-        sm_chunk(std::integral_constant<int, 2>{});
-        __builtin_amdgcn_sched_barrier(0);
-        // g3
-        if (HAS_P2C) { TDB_MF(t3, fr[3][0], kn[0][0]); TDB_MF(t3, fr[3][1], kn[0][1]); }
-        sm_chunk(std::integral_constant<int, 3>{});
-        if (HAS_C2P) put_c(1, t1);
-        __builtin_amdgcn_sched_barrier(0);
-        // g4
-        if (HAS_P2C) { TDB_MF(t3, fr[3][2], kn[0][2]); TDB_MF(t3, fr[3][3], kn[0][3]); TDB_MF(t4, fr[3][0], kn[1][0]); }
-        sm_chunk(std::integral_constant<int, 4>{});
-        if (HAS_C2P) put_c(2, t2);
-        __builtin_amdgcn_sched_barrier(0);
-        // g5
-        if (HAS_P2C) { TDB_MF(t4, fr[3][1], kn[1][1]); TDB_MF(t4, fr[3][2], kn[1][2]); }
-        sm_chunk(std::integral_constant<int, 5>{});
-        __builtin_amdgcn_sched_barrier(0);
-        // g6
-        if (HAS_P2C) { TDB_MF(t4, fr[3][3], kn[1][3]); TDB_MF(t5, fr[4][0], fr[5][0]); TDB_MF(t5, fr[4][1], fr[5][1]); }
-        sm_chunk(std::integral_constant<int, 6>{});
-        if (HAS_P2C) put_p(w, 0, t3);
-        __builtin_amdgcn_sched_barrier(0);
-        // g7
-        if (HAS_P2C) { TDB_MF(t5, fr[4][2], fr[5][2]); TDB_MF(t5, fr[4][3], fr[5][3]); }
-        sm_chunk(std::integral_constant<int, 7>{});
-        __builtin_amdgcn_sched_barrier(0);
-#undef TDB_MF
+        for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+            for (int c = 0; c < 2; ++c) {
+                uint32_t pw[4];
+#pragma unroll
+                for (int h2 = 0; h2 < 4; ++h2) {
+                    const float p0 = __builtin_amdgcn_exp2f(fmaf(s_acc[jt][8 * c + 2 * h2], c_exp, -mc));
+                    const float p1 = __builtin_amdgcn_exp2f(fmaf(s_acc[jt][8 * c + 2 * h2 + 1], c_exp, -mc));
+                    const bf16x2 pr = {(__bf16)p0, (__bf16)p1};
+                    psum = __builtin_amdgcn_fdot2_f32_bf16(pr, ones, psum, false);   // sum of what the MFMA will see
+                    pw[h2] = __builtin_bit_cast(uint32_t, pr);
+                }
+                const bf16x8 pb = __builtin_bit_cast(bf16x8, u32x4{pw[0], pw[1], pw[2], pw[3]});
+                // O^T += V^T.P^T
+#pragma unroll
+                for (int dt = 0; dt < 2; ++dt)
+                    o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[jt][c][dt], pb, o_acc[dt], 0, 0, 0);
+            }
         l_run += psum;
-        if (HAS_P2C) {
-            put_p(w, 1, t4);
-            put_p(4 + (w >> 1), w & 1, t5);
-        }
         TDB_TICK(3);
     };
 
     // steps run in pairs so that the two sets of K fragment registers just swap roles
-    int off = 0;                          // ring slot of window row 0 of the current step
-    auto next_off = [&]() { off = off >= BN ? off - BN : off + WIN - BN; return off; };
-    const int nfull = len / BN;           // steps that need no key mask
     int s = 0;
     for (; s + 1 < nfull; s += 2) {
-        key_step(s, next_off(), kf, kf2, std::false_type{});
-        key_step(s + 1, next_off(), kf2, kf, std::false_type{});
+        key_step(s, kf, kf2, std::false_type{});
+        key_step(s + 1, kf2, kf, std::false_type{});
     }
     if (s < nfull) {
-        key_step(s, next_off(), kf, kf2, std::false_type{});
-        if (nfull < nsteps) key_step(nfull, next_off(), kf2, kf, std::true_type{});
+        key_step(s, kf, kf2, std::false_type{});
+        if (nfull < nsteps) key_step(nfull, kf2, kf, std::true_type{});
     } else if (nfull < nsteps) {
-        key_step(nfull, next_off(), kf, kf2, std::true_type{});
+        key_step(nfull, kf, kf2, std::true_type{});
     }
-    pv_product();                         // of the last step
 
     // ---- epilogue: normalise and store O[i][d]; lane holds d = 32*dt + 8*a + 4*hh + 0..3 of query row il ------
     const float l_tot = l_run + __shfl_xor(l_run, 32);
@@ -572,13 +525,20 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(const TdbKernelParams p)
 }  // namespace
 
 bool tdb_mfma_supported(const TdbKernelParams& p, int dtype) {
-    // bf16, head_dim 64, position terms as fused tables (or none); strips go to the generic kernel
-    return dtype == TDB_BF16 && p.D == 64 && !p.c2p && !p.p2c;
+    // bf16, head_dim 64, position terms as fused tables (or none); strips go to the generic kernel.
+    // Buffer loads address rows with 32-bit byte offsets from the start of a (sequence, head).
+    if (dtype != TDB_BF16 || p.D != 64 || p.c2p || p.p2c) return false;
+    const int64_t lim = int64_t(1) << 31;
+    const int64_t rows = p.L;
+    if (rows * p.ks_l * 2 >= lim || rows * p.vs_l * 2 >= lim) return false;
+    if (p.pk && int64_t(2) * p.span * p.pks_r * 2 >= lim) return false;
+    if (p.pq && int64_t(2) * p.span * p.pqs_r * 2 >= lim) return false;
+    return true;
 }
 
 hipError_t tdb_launch_mfma(const TdbKernelParams& p, int, hipStream_t stream) {
     const int tiles = p.varlen ? p.total / BM + p.B : p.B * ((p.L + BM - 1) / BM);
-    const dim3 grid(tiles, p.H), block(256);
+    const dim3 grid(tiles, p.H), block(NTHREADS);
     const size_t smem = sizeof(Smem);
     const bool c2p = p.pk != nullptr, p2c = p.pq != nullptr;
 #define TDB_LAUNCH(A, B)                                                                                        \
