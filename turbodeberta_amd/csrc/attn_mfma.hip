@@ -38,21 +38,6 @@ typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 
 #define TDB_LDS(T, p) ((__attribute__((address_space(3))) T*)(p))
 
-// Phase timing for development builds (-DTDB_TIMING): one wave accumulates cycle counts per phase.
-#ifdef TDB_TIMING
-__device__ long long tdb_timing[16];
-#define TDB_T0(t) long long tdb_t = clock64(); const bool tdb_on = blockIdx.x == 7 && blockIdx.y == 3 && threadIdx.x == (t)
-#define TDB_TICK(k)                                        \
-    do {                                                   \
-        const long long n_ = clock64();                    \
-        if (tdb_on) tdb_timing[k] += n_ - tdb_t;           \
-        tdb_t = n_;                                        \
-    } while (0)
-#else
-#define TDB_T0(t) do {} while (0)
-#define TDB_TICK(k) do {} while (0)
-#endif
-
 constexpr int BM = TDB_MFMA_TILE;   // query rows per workgroup
 constexpr int BN = 64;              // keys per step
 constexpr int D = 64;
@@ -64,7 +49,7 @@ constexpr int PS = 196;             // row stride of the p2c scratch            
 constexpr int RSRC_FLAGS = 0x00020000;   // raw buffer resource, 32-bit data format
 
 struct Smem {
-    uint16_t k[BN * RS];
+    uint16_t k[2][BN * RS];             // keys of step s live in k[s & 1]
     uint16_t v[BN * RS];
     uint16_t kr[WIN * RS];
     uint16_t qr[WIN * RS];
@@ -120,6 +105,13 @@ __device__ __forceinline__ void lds_wait(uint32_t (&g)[16]) {
                  :
                  : "memory");
 }
+// Workgroup barrier that instruction scheduling may not move anything across either: register-only work (MFMAs,
+// address arithmetic) stays in the pipeline half it was written in.
+__device__ __forceinline__ void phase_barrier() {
+    __builtin_amdgcn_sched_barrier(0);
+    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
+}
 __device__ __forceinline__ uint32_t lds_addr(const void* p) {
     return uint32_t(uintptr_t(TDB_LDS(const char, p)));
 }
@@ -174,24 +166,26 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     // window slides down by 64, so only its 64 lowest positions are fetched and they overwrite the 64 highest
     // of the previous step.  Window row x of step s sits in ring slot (x + off_s) mod 192, off_s = (128*s) mod 192.
     //
-    // Each step has two halves separated by workgroup barriers:
+    // Each step has two halves separated by workgroup barriers, arranged so that in either half one role is on
+    // the LDS and the other on the matrix cores:
     //   A  score waves read this step's position terms out of the C'/P' scratch into their score accumulators;
-    //      position waves hand their register-prefetched global data to LDS: keys of step s+1, values of step s,
-    //      64 window rows of step s+1;
+    //      position waves hand register-prefetched global data to LDS (keys of step s+2, values of step s, 64 window
+    //      rows of step s+2) and run the 24 position MFMAs of step s+1 on fragments they already hold;
     //   B  score waves: S^T(s), softmax(s), P.V(s), and they pick up the K fragments of step s+1;
-    //      position waves: global fetches for the next half A, then the position products C', P' of step s+1 into
-    //      the now free scratch.
+    //      position waves: results of step s+1 into the now free scratch, global fetches for the next half A,
+    //      LDS fragments of step s+2.
     const int nsteps = (len + BN - 1) / BN;
     const int nfull = len / BN;           // steps that need no key mask
-    int off = 0;                          // ring slot of window row 0 of the current step
-    auto next_off = [&]() { off = off >= BN ? off - BN : off + WIN - BN; return off; };
     const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    auto prev_off = [](int o) { return o >= BN ? o - BN : o + WIN - BN; };   // ring offset of the following step
 
-    // prologue, all 512 threads: keys and whole window of step 0 to LDS
+    // prologue, all 512 threads: keys of steps 0 and 1 and the whole window of step 0 to LDS
     {
         const int row = tid >> 3, ch = tid & 7;              // rows 0..63
-        *reinterpret_cast<u32x4*>(&sm.k[row * RS + ch * 8]) =
+        *reinterpret_cast<u32x4*>(&sm.k[0][row * RS + ch * 8]) =
             *reinterpret_cast<const u32x4*>(K + int64_t(min(row, len - 1)) * p.ks_l + ch * 8);
+        *reinterpret_cast<u32x4*>(&sm.k[1][row * RS + ch * 8]) =
+            *reinterpret_cast<const u32x4*>(K + int64_t(min(BN + row, len - 1)) * p.ks_l + ch * 8);
         if (HAS_POS) {
 #pragma unroll
             for (int n = 0; n < WIN / 64; ++n) {
@@ -209,7 +203,6 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     if (!score_role) {
         // ================================================= position waves ==========================================
         const int stid = tid - 256;
-        TDB_T0(320);
         const int srow = stid >> 3, sch = stid & 7;          // this thread stages rows srow, srow+32 (chunk sch)
         // global -> registers through buffer loads.  The buffer of a step starts at its first row and ends with the
         // last row of the sequence, so rows past the end come back as zeros (hardware range check) with no lane
@@ -247,41 +240,26 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
                 for (int n = 0; n < 2; ++n) dl_next[n] = delta_of(row0 - BN * s - (BN - 1) + srow + 32 * n);
             }
         };
-        auto store = [&](int o) {              // registers -> LDS
+        auto store = [&](int o, int kbuf) {    // registers -> LDS: keys into k[kbuf], window rows at ring offset o
 #pragma unroll
             for (int n = 0; n < 2; ++n) {
                 const int r = srow + 32 * n;
-                *reinterpret_cast<u32x4*>(&sm.k[r * RS + sch * 8]) = pre_k[n];
+                *reinterpret_cast<u32x4*>(&sm.k[kbuf][r * RS + sch * 8]) = pre_k[n];
                 *reinterpret_cast<u32x4*>(&sm.v[r * RS + sch * 8]) = pre_v[n];
                 if (HAS_C2P) *reinterpret_cast<u32x4*>(&sm.kr[(o + r) * RS + sch * 8]) = pre_kr[n];
                 if (HAS_P2C) *reinterpret_cast<u32x4*>(&sm.qr[(o + r) * RS + sch * 8]) = pre_qr[n];
             }
         };
-        // Position products of one key step from the ring at offset o and the keys in sm.k, into the scratch:
-        //   c2p  C'^T[r, i] = K_r'[r].Q_i over the 96-position sub-window of query block w, stored as fp32 C'[i][r'];
-        //   p2c  P'^T[r, j] = Q_r'[r].K_j over the whole window (6 x 2 tiles): wave w takes position tile w against
-        //        both key tiles and tile (4 + w/2, w&1); stored as bf16 P'[j][r''].
-        auto pos_products = [&](int o) {
+        // Position products of one key step, in three stages that the pipeline places in different halves:
+        //   load_frags  MFMA operands out of LDS: K_r' rows of the 96-position sub-window of query block w (fr),
+        //               Q_r' rows of position tiles w and 4 + w/2 of the workgroup window (fq), both key tiles (kb);
+        //   products    c2p  C'^T[r, i] = K_r'[r].Q_i  (3 tiles),  p2c  P'^T[r, j] = Q_r'[r].K_j  (wave w: tile w
+        //               against both key tiles, and tile (4 + w/2, w & 1)) -- 24 MFMAs;
+        //   put_results c2p as fp32 C'[i][r'], p2c as bf16 P'[j][r''] into the scratch.
+        bf16x8 fr[3][4], fq[2][4], kb[2][4];
+        f32x16 res[6];
+        auto load_frags = [&](int o, int kbuf) {
             auto ring = [&](int x) { const int t = x + o; return t >= WIN ? t - WIN : t; };
-            auto chain = [&](const bf16x8 (&a)[4], const bf16x8 (&bb)[4]) {
-                f32x16 acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], bb[0], zero16, 0, 0, 0);
-#pragma unroll
-                for (int c = 1; c < 4; ++c) acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[c], bb[c], acc, 0, 0, 0);
-                return acc;
-            };
-            auto put_c = [&](int rt, const f32x16& acc) {
-#pragma unroll
-                for (int a = 0; a < 4; ++a)
-                    *reinterpret_cast<float4*>(&sm.c[w][il * CS + 32 * rt + 8 * a + 4 * hh]) =
-                        float4{acc[4 * a], acc[4 * a + 1], acc[4 * a + 2], acc[4 * a + 3]};
-            };
-            auto put_p = [&](int rt, int jt, const f32x16& acc) {
-#pragma unroll
-                for (int a = 0; a < 4; ++a)
-                    *reinterpret_cast<u32x2*>(&sm.p[(32 * jt + il) * PS + 32 * rt + 8 * a + 4 * hh]) =
-                        pack4(acc[4 * a], acc[4 * a + 1], acc[4 * a + 2], acc[4 * a + 3]);
-            };
-            bf16x8 fr[3][4], fq[2][4], kb[3][4];
             if (HAS_C2P) {
 #pragma unroll
                 for (int rt = 0; rt < 3; ++rt) {
@@ -296,60 +274,93 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
                 for (int c = 0; c < 4; ++c) {
                     fq[0][c] = lds_frag(sm.qr, row3, 16 * c + 8 * hh);
                     fq[1][c] = lds_frag(sm.qr, row4, 16 * c + 8 * hh);
-                    kb[0][c] = lds_frag(sm.k, il, 16 * c + 8 * hh);
-                    kb[1][c] = lds_frag(sm.k, 32 + il, 16 * c + 8 * hh);
+                    kb[0][c] = lds_frag(sm.k[kbuf], il, 16 * c + 8 * hh);
+                    kb[1][c] = lds_frag(sm.k[kbuf], 32 + il, 16 * c + 8 * hh);
                 }
             }
-            // every fragment read is in flight before the first MFMA waits for one
-            __builtin_amdgcn_sched_barrier(0);
-            TDB_TICK(8);
+        };
+        auto products = [&]() {
+            auto chain = [&](const bf16x8 (&a)[4], const bf16x8 (&bb)[4]) {
+                f32x16 acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], bb[0], zero16, 0, 0, 0);
+#pragma unroll
+                for (int c = 1; c < 4; ++c) acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[c], bb[c], acc, 0, 0, 0);
+                return acc;
+            };
+            if (HAS_C2P) {
+#pragma unroll
+                for (int rt = 0; rt < 3; ++rt) res[rt] = chain(fr[rt], qb);
+            }
             if (HAS_P2C) {
+                bf16x8 kx[4];
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {   // key tile (w & 1), chosen without indexing registers
                     const u32x4 x0 = __builtin_bit_cast(u32x4, kb[0][c]), x1 = __builtin_bit_cast(u32x4, kb[1][c]);
                     u32x4 r;
 #pragma unroll
                     for (int e = 0; e < 4; ++e) r[e] = (w & 1) ? x1[e] : x0[e];
-                    kb[2][c] = __builtin_bit_cast(bf16x8, r);
+                    kx[c] = __builtin_bit_cast(bf16x8, r);
                 }
+                res[3] = chain(fq[0], kb[0]);
+                res[4] = chain(fq[0], kb[1]);
+                res[5] = chain(fq[1], kx);
             }
+        };
+        auto put_results = [&]() {
             if (HAS_C2P) {
-                const f32x16 a0 = chain(fr[0], qb);
-                const f32x16 a1 = chain(fr[1], qb);
-                put_c(0, a0);
-                const f32x16 a2 = chain(fr[2], qb);
-                put_c(1, a1);
-                put_c(2, a2);
+#pragma unroll
+                for (int rt = 0; rt < 3; ++rt)
+#pragma unroll
+                    for (int a = 0; a < 4; ++a)
+                        *reinterpret_cast<float4*>(&sm.c[w][il * CS + 32 * rt + 8 * a + 4 * hh]) =
+                            float4{res[rt][4 * a], res[rt][4 * a + 1], res[rt][4 * a + 2], res[rt][4 * a + 3]};
             }
-            TDB_TICK(9);
             if (HAS_P2C) {
-                const f32x16 a0 = chain(fq[0], kb[0]);
-                const f32x16 a1 = chain(fq[0], kb[1]);
-                put_p(w, 0, a0);
-                const f32x16 a2 = chain(fq[1], kb[2]);
-                put_p(w, 1, a1);
-                put_p(4 + (w >> 1), w & 1, a2);
+                auto put_p = [&](int rt, int jt, const f32x16& acc) {
+#pragma unroll
+                    for (int a = 0; a < 4; ++a)
+                        *reinterpret_cast<u32x2*>(&sm.p[(32 * jt + il) * PS + 32 * rt + 8 * a + 4 * hh]) =
+                            pack4(acc[4 * a], acc[4 * a + 1], acc[4 * a + 2], acc[4 * a + 3]);
+                };
+                put_p(w, 0, res[3]);
+                put_p(w, 1, res[4]);
+                put_p(4 + (w >> 1), w & 1, res[5]);
             }
         };
 
+        // prologue: products of step 0; window rows of step 1 (they overwrite rows step 0 is done with);
+        // fragments of step 1; prefetch for half A of step 0
+        const int off1 = prev_off(0);
         fetch_delta(1);
-        fetch(1, 0);
+        load_frags(0, 0);
+        products();
+        put_results();
+        fetch(2, 0);                      // pre_k: keys of step 2 (unused rows of step 1), pre_v: values of step 0
+        phase_barrier();                  // every position wave has its fragments of step 0
+        if (HAS_POS) {
+#pragma unroll
+            for (int n = 0; n < 2; ++n) {
+                const int r = srow + 32 * n;
+                if (HAS_C2P) *reinterpret_cast<u32x4*>(&sm.kr[(off1 + r) * RS + sch * 8]) = pre_kr[n];
+                if (HAS_P2C) *reinterpret_cast<u32x4*>(&sm.qr[(off1 + r) * RS + sch * 8]) = pre_qr[n];
+            }
+        }
         fetch_delta(2);
-        pos_products(0);
-        TDB_TICK(11);
+        phase_barrier();                  // window of step 1 complete
+        load_frags(off1, 1);
+        fetch(2, 0);                      // keys of step 2, values of step 0, window rows of step 2
+        fetch_delta(3);
+        int off2 = prev_off(off1);        // ring offset of step s+2
         for (int s = 0; s < nsteps; ++s) {
-            const int off_next = next_off();
-            __syncthreads();              // scratch of step s complete
-            TDB_TICK(4);
-            store(off_next);              // keys of step s+1, values of step s, new window rows of step s+1
-            TDB_TICK(5);
-            __syncthreads();              // scratch is free again; the staged tiles are visible
-            TDB_TICK(6);
-            fetch(s + 2, s + 1);
-            fetch_delta(s + 3);
-            TDB_TICK(7);
-            pos_products(off_next);       // of step s+1 (harmless left-over work in the last step)
-            TDB_TICK(10);
+            phase_barrier();              // scratch of step s complete
+            products();                   // of step s+1, into registers; issued first: the wait for the
+            __builtin_amdgcn_sched_barrier(0);  // prefetched global data then passes under the MFMAs
+            store(off2, s & 1);           // keys of step s+2, values of step s, new window rows of step s+2
+            phase_barrier();              // score waves are done with the scratch; the staged tiles are visible
+            put_results();                // of step s+1 (harmless left-over work in the last step)
+            fetch(s + 3, s + 1);
+            fetch_delta(s + 4);
+            load_frags(off2, s & 1);      // of step s+2
+            off2 = prev_off(off2);
         }
         return;
     }
@@ -361,20 +372,19 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
 
     bf16x8 kf[2][4], kf2[2][4];           // K fragments: A operand of S^T = K.Q^T; two sets that swap roles
-    auto load_kf = [&](bf16x8 (&dst)[2][4]) {
+    auto load_kf = [&](bf16x8 (&dst)[2][4], int kbuf) {
 #pragma unroll
         for (int jt = 0; jt < 2; ++jt)
 #pragma unroll
-            for (int c = 0; c < 4; ++c) dst[jt][c] = lds_frag(sm.k, 32 * jt + il, 16 * c + 8 * hh);
+            for (int c = 0; c < 4; ++c) dst[jt][c] = lds_frag(sm.k[kbuf], 32 * jt + il, 16 * c + 8 * hh);
     };
-    load_kf(kf);
-
-    TDB_T0(64);
+    load_kf(kf, 0);
+    phase_barrier();                      // the two prologue barriers of the position waves
+    phase_barrier();
     // One key step.  MASKED: the step reaches past the end of the sequence (only the last step can).
     auto key_step = [&](int s, const bf16x8 (&kc)[2][4], bf16x8 (&kn)[2][4], auto masked_tag) {
         constexpr bool MASKED = decltype(masked_tag)::value;
-        __syncthreads();                  // scratch of step s complete
-        TDB_TICK(0);
+        phase_barrier();                  // scratch of step s complete
 
         // ---- half A: position terms of step s out of the scratch.  Element (jj, i) of the score tile takes
         //      C'[i][i-jj+63] (fp32, straight into the accumulator) and P'[jj][32w+i-jj+63] (bf16) ----------------
@@ -411,16 +421,14 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
                 for (int e = 0; e < 16; ++e)   // bf16 pair (value, 0) . (1, 1) + acc
                     s_acc[jt][e] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, g[jt][e]), ones, s_acc[jt][e], false);
         }
-        TDB_TICK(1);
-        __syncthreads();                  // scratch is free again; keys of step s+1 and values of step s are staged
-        TDB_TICK(2);
+        phase_barrier();                  // scratch is free again; keys of step s+1 and values of step s are staged
 
         // ---- half B ---------------------------------------------------------------------------------------------
 #pragma unroll
         for (int c = 0; c < 4; ++c)
 #pragma unroll
             for (int jt = 0; jt < 2; ++jt) s_acc[jt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kc[jt][c], qb[c], s_acc[jt], 0, 0, 0);
-        load_kf(kn);                      // K fragments of step s+1
+        load_kf(kn, (s + 1) & 1);         // K fragments of step s+1
         // V^T fragments through the transposing LDS read: the lane provides the address of 4 dims of one key
         bf16x8 vf[2][2][2];               // [key tile][16-key chunk][dim tile]
         {
@@ -490,7 +498,6 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
                     o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[jt][c][dt], pb, o_acc[dt], 0, 0, 0);
             }
         l_run += psum;
-        TDB_TICK(3);
     };
 
     // steps run in pairs so that the two sets of K fragment registers just swap roles
