@@ -44,7 +44,11 @@ hipError_t tdb_launch_generic(const TdbKernelParams& p, int dtype, hipStream_t s
 hipError_t tdb_launch_mfma(const TdbKernelParams& p, int dtype, hipStream_t stream);
 
 // Maps blockIdx.x to (sequence, first row of the tile, valid length).  Returns false when the
-// block has no tile (packed launches are sized by an upper bound on the tile count).
+// block has no tile (packed launches are sized by an upper bound on the tile count).  Must be
+// called by whole waves with identical arguments.  For packed input the wave scans cu_seqlens 64
+// sequences at a time: one load per lane, a prefix sum of the per-sequence tile counts across the
+// wave, and a ballot to pick the sequence that owns tile `block` -- no serial chain of dependent
+// loads, and no work list built on the host.
 __device__ __forceinline__ bool tdb_locate_tile(const TdbKernelParams& p, int tile_rows, int block,
                                                 int& b, int& row0, int& len, int64_t& tok0) {
     if (!p.varlen) {
@@ -55,20 +59,37 @@ __device__ __forceinline__ bool tdb_locate_tile(const TdbKernelParams& p, int ti
         tok0 = 0;
         return true;
     }
+    const int lane = threadIdx.x & 63;
     int t = block;
-    for (b = 0; b < p.B; ++b) {
-        const int s = p.cu_seqlens[b], e = p.cu_seqlens[b + 1];
-        int n = e - s;
-        if (s < 0 || n < 0 || e > p.total) n = 0;       // malformed entry: no tiles
-        n = min(n, p.L);
+    for (int b0 = 0; b0 < p.B; b0 += 64) {
+        const int bb = b0 + lane;
+        int s = 0, n = 0;
+        if (bb < p.B) {
+            s = p.cu_seqlens[bb];
+            const int e = p.cu_seqlens[bb + 1];
+            n = e - s;
+            if (s < 0 || n < 0 || e > p.total) n = 0;   // malformed entry: no tiles
+            n = min(n, p.L);
+        }
         const int nt = (n + tile_rows - 1) / tile_rows;
-        if (t < nt) {
-            row0 = t * tile_rows;
-            len = n;
-            tok0 = s;
+        int incl = nt;                                   // inclusive prefix sum over the wave
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const int up = __shfl_up(incl, d);
+            if (lane >= d) incl += up;
+        }
+        const int chunk_tiles = __builtin_amdgcn_readlane(incl, 63);
+        if (t < chunk_tiles) {
+            const unsigned long long owners = __builtin_amdgcn_ballot_w64(incl > t);
+            const int ln = __builtin_amdgcn_readfirstlane(__builtin_ctzll(owners));
+            const int before = __builtin_amdgcn_readlane(incl, ln) - __builtin_amdgcn_readlane(nt, ln);
+            b = b0 + ln;
+            row0 = (t - before) * tile_rows;
+            len = __builtin_amdgcn_readlane(n, ln);
+            tok0 = __builtin_amdgcn_readlane(s, ln);
             return true;
         }
-        t -= nt;
+        t -= chunk_tiles;
     }
     return false;
 }
