@@ -1,0 +1,142 @@
+"""The Hugging Face patch glue and the packing helpers.
+
+CPU part: parameter names equal Hugging Face's (stock checkpoints load), in-place patching, mask
+reduction, packing round trips, loud failure without a GPU.  GPU part: a two-layer model against
+the golden last hidden state written by Hugging Face's eager model, the eager fallback for
+``output_attentions``, and a bf16 encoder against Hugging Face eager run on the same device."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+transformers = pytest.importorskip("transformers")
+from transformers import DebertaV2Config  # noqa: E402
+from transformers.models.deberta_v2.modeling_deberta_v2 import DebertaV2Model, DisentangledSelfAttention  # noqa: E402
+
+from golden_inputs import fill_params, tiny_model_config, tiny_model_inputs  # noqa: E402
+from turbodeberta_amd import padding  # noqa: E402
+from turbodeberta_amd.model import (FlashDebertaV2Model, FlashDisentangledSelfAttention, patch_model)  # noqa: E402
+
+
+def _tiny():
+    return DebertaV2Config(**tiny_model_config())
+
+
+def test_parameter_names_match_hugging_face():
+    ours, theirs = FlashDebertaV2Model(_tiny()), DebertaV2Model(_tiny())
+    assert list(ours.state_dict()) == list(theirs.state_dict())
+    ours.load_state_dict(theirs.state_dict(), strict=True)
+    assert sum(isinstance(m, FlashDisentangledSelfAttention) for m in ours.modules()) == 2
+
+
+def test_patch_model_in_place():
+    m = DebertaV2Model(_tiny())
+    before = {k: v.clone() for k, v in m.state_dict().items()}
+    assert patch_model(m) is m
+    assert all(type(x) is not DisentangledSelfAttention for x in m.modules())
+    assert sum(isinstance(x, FlashDisentangledSelfAttention) for x in m.modules()) == 2
+    assert all(torch.equal(v, before[k]) for k, v in m.state_dict().items())
+
+
+def test_forward_without_gpu_fails_loudly():
+    m = FlashDebertaV2Model(_tiny()).eval()
+    ids, mask = tiny_model_inputs()
+    with pytest.raises(RuntimeError, match="no CPU implementation"):
+        with torch.no_grad():
+            m(input_ids=torch.from_numpy(ids), attention_mask=torch.from_numpy(mask))
+
+
+def test_key_padding_mask_and_unpad_data():
+    m2 = torch.tensor([[1, 1, 1, 0, 0], [1, 1, 1, 1, 1], [1, 0, 0, 0, 0]])
+    ext = m2.unsqueeze(1).unsqueeze(2)
+    m4 = ext * ext.squeeze(-2).unsqueeze(-1)                      # what the HF encoder builds
+    for m in (m2, m4, m4[:, 0]):
+        assert torch.equal(padding.key_padding_mask(m), m2)
+        assert padding.sequence_lengths(m).tolist() == [3, 5, 1]
+    idx, cu, mx = padding._get_unpad_data(m4)
+    assert cu.dtype == torch.int32 and cu.tolist() == [0, 3, 8, 9] and mx == 5
+    assert idx.tolist() == [0, 1, 2, 5, 6, 7, 8, 9, 10]
+
+
+def test_pack_unpack_round_trip():
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(3, 5, 2, 4, generator=g)
+    m2 = torch.tensor([[1, 1, 1, 0, 0], [1, 1, 1, 1, 1], [1, 0, 0, 0, 0]])
+    packed, idx, cu, mx = padding.unpad_input(x, m2)
+    assert packed.shape == (9, 2, 4) and torch.equal(packed[3:8], x[1])
+    back = padding.pad_input(packed, idx, 3, 5)
+    assert torch.equal(back, x * m2[:, :, None, None])
+    q, k, v, pk, pq, idx2, (cq, ck), (mq, mk) = padding._upad_input(x, x, x, None, None, m2, 5, 2)
+    assert torch.equal(q, packed) and pk is None and torch.equal(cq, cu) and mq == 5
+
+
+# ------------------------------------------------------------------------------------- GPU
+
+@pytest.mark.gpu
+def test_tiny_model_matches_hf_golden(golden_dir):
+    cfg = _tiny()
+    model = FlashDebertaV2Model(cfg).eval()
+    fill_params(model)
+    model = model.to("cuda:0")
+    ids, mask = tiny_model_inputs()
+    gold = torch.from_numpy(np.load(os.path.join(golden_dir, "hf_tiny_model.npz"))["last_hidden_state"])
+    print("[case] tiny model fp32", flush=True)
+    with torch.no_grad():
+        out = model(input_ids=torch.from_numpy(ids).cuda(), attention_mask=torch.from_numpy(mask).cuda()).last_hidden_state
+    out = out.float().cpu()
+    valid = torch.from_numpy(mask).bool()
+    rel = (out[valid] - gold[valid]).abs().max() / gold[valid].abs().max()
+    assert rel <= 1e-4, rel
+
+
+@pytest.mark.gpu
+def test_output_attentions_falls_back_to_eager():
+    cfg = _tiny()
+    ours, theirs = FlashDebertaV2Model(cfg).eval(), DebertaV2Model(cfg).eval()
+    fill_params(ours)
+    theirs.load_state_dict(ours.state_dict())
+    ours, theirs = ours.cuda(), theirs.cuda()
+    ids, mask = tiny_model_inputs()
+    ids, mask = torch.from_numpy(ids).cuda(), torch.from_numpy(mask).cuda()
+    with torch.no_grad():
+        a = ours(input_ids=ids, attention_mask=mask, output_attentions=True)
+        b = theirs(input_ids=ids, attention_mask=mask, output_attentions=True)
+    assert len(a.attentions) == 2 and torch.allclose(a.attentions[0], b.attentions[0], atol=1e-5)
+    assert torch.allclose(a.last_hidden_state, b.last_hidden_state, atol=1e-4)
+
+
+@pytest.mark.gpu
+def test_bf16_encoder_matches_hf_eager_on_device():
+    # v3-base-like widths, 3 layers: patched model vs the unpatched Hugging Face model, both bf16 on the GPU
+    cfg = DebertaV2Config(vocab_size=1000, hidden_size=768, num_hidden_layers=3, num_attention_heads=12,
+                          intermediate_size=3072, hidden_dropout_prob=0.0, attention_probs_dropout_prob=0.0,
+                          max_position_embeddings=512, type_vocab_size=0, relative_attention=True, position_buckets=256,
+                          max_relative_positions=512, share_att_key=True, pos_att_type=["c2p", "p2c"],
+                          norm_rel_ebd="layer_norm", position_biased_input=False, layer_norm_eps=1e-7)
+    torch.manual_seed(0)
+    truth = DebertaV2Model(cfg).eval()
+    fill_params(truth, seed=5)
+    theirs = DebertaV2Model(cfg).eval()
+    theirs.load_state_dict(truth.state_dict())
+    ours = patch_model(DebertaV2Model(cfg).eval())
+    ours.load_state_dict(truth.state_dict())
+    truth = truth.to("cuda:0")                                            # float32 eager: the yardstick
+    theirs, ours = theirs.to("cuda:0", torch.bfloat16), ours.to("cuda:0", torch.bfloat16)
+    rs = np.random.RandomState(1)
+    lens = np.array([300, 128, 77, 299])
+    ids = torch.from_numpy(rs.randint(1, 1000, size=(4, 300))).cuda()
+    mask = torch.from_numpy((np.arange(300)[None] < lens[:, None]).astype(np.int64)).cuda()
+    print("[case] bf16 3-layer encoder", flush=True)
+    with torch.no_grad():
+        a = ours(input_ids=ids, attention_mask=mask).last_hidden_state.float()
+        b = theirs(input_ids=ids, attention_mask=mask).last_hidden_state.float()
+        t = truth(input_ids=ids, attention_mask=mask).last_hidden_state
+    valid = mask.bool()
+    # Hidden states are LayerNorm outputs of order 1, so one bf16 ulp is 8e-3.  The patched model must be as close
+    # to the float32 model as Hugging Face's own bf16 eager run is (it keeps fp32 scores, so it is usually closer).
+    err_ours = (a[valid] - t[valid]).abs()
+    err_hf = (b[valid] - t[valid]).abs()
+    assert err_ours.mean().item() <= 1.25 * err_hf.mean().item() + 1e-4, (err_ours.mean().item(), err_hf.mean().item())
+    assert err_ours.max().item() <= 1.5 * err_hf.max().item() + 1e-3, (err_ours.max().item(), err_hf.max().item())
+    assert (a[valid] - b[valid]).abs().max().item() <= 1e-1
