@@ -147,6 +147,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--workload", choices=["both", "fixed", "varlen"], default="both")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also launch one plain device copy of 512 MiB (read) + 512 MiB (write), the yardstick the "
+                         "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: every figure of this path is per GPU (no collectives); run with --gpus 1",
@@ -157,6 +160,13 @@ def main():
         sys.exit(2)
     dev = torch.device("cuda", int(os.environ.get("LOCAL_RANK", "0")))
     torch.cuda.set_device(dev)
+
+    if args.calibrate_copy:
+        src = torch.zeros(256 * 1024 * 1024, dtype=torch.bfloat16, device=dev)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     out = {"metric": METRIC, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic"}
