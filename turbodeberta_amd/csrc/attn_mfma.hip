@@ -47,6 +47,7 @@ constexpr int RS = 72;              // LDS row stride (elements) of 64-wide bf16
 constexpr int CS = 100;             // row stride (floats) of the per-block c2p scratch [32][96 used]
 constexpr int PS = 196;             // row stride of the p2c scratch                   [64][192 used]
 constexpr int RSRC_FLAGS = 0x00020000;   // raw buffer resource, 32-bit data format
+constexpr int XCD_GROUP = 4;        // query tiles of one (sequence, head) kept on one XCD
 
 struct Smem {
     uint16_t k[2][BN * RS];             // keys of step s live in k[s & 1]
@@ -127,11 +128,22 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     const bool score_role = wave < 4;     // waves 0..3 score, 4..7 position; wave w and w+4 share query block w
     const int w = wave & 3, l = tid & 63;
     const int il = l & 31, hh = l >> 5;
-    const int head = blockIdx.y;
+    // Workgroup -> (tile, head).  Consecutive workgroup ids go round-robin over the 8 XCDs, each with its own L2.
+    // The launch is 1-D and ids are regrouped so that XCD_GROUP tiles that are neighbours along the query axis --
+    // the tiles that read the same K and V -- run on one XCD and fetch K / V from HBM once instead of once each.
+    const int tiles_x = p.varlen ? p.total / BM + p.B : p.B * ((p.L + BM - 1) / BM);
+    int tile_id, head;
+    {
+        const int n = blockIdx.x, xcd = n & 7, slot = n >> 3;
+        const int v = ((slot / XCD_GROUP) * 8 + xcd) * XCD_GROUP + slot % XCD_GROUP;
+        if (v >= tiles_x * p.H) return;
+        head = v / tiles_x;
+        tile_id = v - head * tiles_x;
+    }
 
     int b, row0, len;
     int64_t tok0;
-    if (!tdb_locate_tile(p, BM, blockIdx.x, b, row0, len, tok0)) return;
+    if (!tdb_locate_tile(p, BM, tile_id, b, row0, len, tok0)) return;
 
     const uint16_t* Q = static_cast<const uint16_t*>(p.q) + (p.varlen ? tok0 * p.qs_l : int64_t(b) * p.qs_b) + int64_t(head) * p.qs_h;
     const uint16_t* K = static_cast<const uint16_t*>(p.k) + (p.varlen ? tok0 * p.ks_l : int64_t(b) * p.ks_b) + int64_t(head) * p.ks_h;
@@ -544,8 +556,9 @@ bool tdb_mfma_supported(const TdbKernelParams& p, int dtype) {
 }
 
 hipError_t tdb_launch_mfma(const TdbKernelParams& p, int, hipStream_t stream) {
-    const int tiles = p.varlen ? p.total / BM + p.B : p.B * ((p.L + BM - 1) / BM);
-    const dim3 grid(tiles, p.H), block(NTHREADS);
+    const int64_t tiles = int64_t(p.varlen ? p.total / BM + p.B : p.B * ((p.L + BM - 1) / BM)) * p.H;
+    const int64_t round = 8 * XCD_GROUP;                 // the id regrouping is a bijection on multiples of this
+    const dim3 grid(unsigned((tiles + round - 1) / round * round)), block(NTHREADS);
     const size_t smem = sizeof(Smem);
     const bool c2p = p.pk != nullptr, p2c = p.pq != nullptr;
 #define TDB_LAUNCH(A, B)                                                                                        \
