@@ -34,6 +34,10 @@ BUCKETS, MAX_REL, SPAN = 256, 512, 256
 PEAK_BF16_TFLOPS = 2500.0       # MI355X dense bf16 MFMA, AMD public spec
 PEAK_HBM_GBS = 8000.0
 METRIC = "attn TFLOP/s + tokens/s, DeBERTa-v3-base b32xL512 bf16, fixed and varlen"
+# HBM bytes per launch from `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` runs of this script, each counter scaled
+# by what it reads for a plain 512 MiB device copy (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000); the runs and raw counter
+# values are recorded in profiles/attn_mfma_kernel_fixed_b32xL512.md and profiles/attn_mfma_kernel_varlen_64seq.md.
+MEASURED_TRAFFIC_BYTES = {"fixed": 103.9e6, "varlen": 138.3e6}
 
 
 def flops_of(lengths) -> float:
@@ -180,9 +184,9 @@ def main():
             "tokens_per_s": round(float(lengths.sum()) / (wall_ms * 1e-3), 1),
             "core_tflops": round(H * sum(4.0 * int(l) ** 2 * D for l in lengths) / (wall_ms * 1e-3) / 1e12, 2),
             "roofline": {"bound": "mfma", "achieved": round(ach, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                         "frac": round(ach / PEAK_BF16_TFLOPS, 4), "traffic": None, "kernel": kernel,
+                         "frac": round(ach / PEAK_BF16_TFLOPS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(name), "kernel": kernel,
                          "kernel_ms_mean": round(mean_ms, 4), "kernel_ms_median": round(med_ms, 4),
-                         "kernel_ms_min": round(min_ms, 4), "algorithmic_gflop": round(fl / 1e9, 3),
+                         "kernel_ms_min": round(min_ms, 4), "algorithmic_gflop": round(fl / 1e9, 3), "algorithmic_bytes": algorithmic_bytes(lengths),
                          "hbm_gbs_algorithmic": round(algorithmic_bytes(lengths) / (mean_ms * 1e-3) / 1e9, 1)},
         }
 
