@@ -108,6 +108,39 @@ __device__ __forceinline__ void lds_wait(uint32_t (&g)[16]) {
 }
 // Workgroup barrier that instruction scheduling may not move anything across either: register-only work (MFMAs,
 // address arithmetic) stays in the pipeline half it was written in.
+#ifdef TDB_TIMING
+// Development aid (off in the library build): cycle stamps of one workgroup's first score wave and first position
+// wave, summed per pipeline phase, and entry / exit wall-clock times of every workgroup.
+__device__ long long tdb_timing[16];
+__device__ long long tdb_ptiming[16];
+__device__ long long tdb_trace[4 * 4096];   // per workgroup: entry, exit (100 MHz wall clock), hardware id, steps
+#define TDB_T_ENTRY const long long t_entry = __builtin_readcyclecounter(); const long long t_wall = wall_clock64(); \
+        long long t_pro[8] = {0, 0, 0, 0, 0, 0, 0, 0}; long long t_plast = t_entry;
+#define TDB_PSTAMP(slot) do { __builtin_amdgcn_sched_barrier(0); const long long t_now = __builtin_readcyclecounter(); \
+        t_pro[slot] += t_now - t_plast; t_plast = t_now; __builtin_amdgcn_sched_barrier(0); } while (0)
+#define TDB_PRESET do { t_plast = __builtin_readcyclecounter(); } while (0)
+#define TDB_P_FLUSH do { if (blockIdx.x == TDB_TIMING && (threadIdx.x & 255) == 0) \
+        for (int t_i = 0; t_i < 8; ++t_i) tdb_ptiming[t_i + (threadIdx.x >> 8) * 8] = t_pro[t_i]; } while (0)
+#define TDB_T_DECL long long t_acc[6] = {0, 0, 0, 0, 0, 0}; long long t_last = __builtin_readcyclecounter(); t_acc[4] = t_last - t_entry;
+#define TDB_STAMP(slot) do { __builtin_amdgcn_sched_barrier(0); const long long t_now = __builtin_readcyclecounter(); \
+        t_acc[slot] += t_now - t_last; t_last = t_now; __builtin_amdgcn_sched_barrier(0); } while (0)
+#define TDB_T_FLUSH(base) do { if (blockIdx.x == TDB_TIMING && (threadIdx.x & 255) == 0) \
+        for (int t_i = 0; t_i < 6; ++t_i) tdb_timing[(base) + t_i] = t_acc[t_i]; } while (0)
+#define TDB_TRACE_EXIT do { if (threadIdx.x == 0 && blockIdx.x < 4096) { \
+        tdb_trace[4 * blockIdx.x] = t_wall; tdb_trace[4 * blockIdx.x + 1] = wall_clock64(); \
+        tdb_trace[4 * blockIdx.x + 2] = (long long)__builtin_amdgcn_s_getreg(63492) | ((long long)__builtin_amdgcn_s_getreg((31 << 11) | 20) << 32); \
+        tdb_trace[4 * blockIdx.x + 3] = nsteps; } } while (0)
+#else
+#define TDB_T_ENTRY
+#define TDB_PSTAMP(slot)
+#define TDB_PRESET
+#define TDB_P_FLUSH
+#define TDB_T_DECL
+#define TDB_STAMP(slot)
+#define TDB_T_FLUSH(base)
+#define TDB_TRACE_EXIT
+#endif
+
 __device__ __forceinline__ void phase_barrier() {
     __builtin_amdgcn_sched_barrier(0);
     __syncthreads();
@@ -118,130 +151,257 @@ __device__ __forceinline__ uint32_t lds_addr(const void* p) {
 }
 
 template <bool HAS_C2P, bool HAS_P2C>
-__global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelParams p) {
+__global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelParams p, const int nblocks) {
     extern __shared__ __attribute__((aligned(16))) char smem_raw[];
     Smem& sm = *reinterpret_cast<Smem*>(smem_raw);
     constexpr bool HAS_POS = HAS_C2P || HAS_P2C;
 
+    TDB_T_ENTRY
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const bool score_role = wave < 4;     // waves 0..3 score, 4..7 position; wave w and w+4 share query block w
     const int w = wave & 3, l = tid & 63;
     const int il = l & 31, hh = l >> 5;
-    // Workgroup -> (tile, head).  Consecutive workgroup ids go round-robin over the 8 XCDs, each with its own L2.
-    // The launch is 1-D and ids are regrouped so that XCD_GROUP tiles that are neighbours along the query axis --
-    // the tiles that read the same K and V -- run on one XCD and fetch K / V from HBM once instead of once each.
+
+    // ---- tiles --------------------------------------------------------------------------------------------------
+    // The workgroup is persistent: the launch has one workgroup per CU (LDS admits no second one), and workgroup g
+    // takes the virtual blocks g, g + gridDim.x, ...  While the last key step of a tile runs, the first LDS stage of
+    // the next tile is already on its way from global memory, so that the chain of dependent global reads that
+    // starts a tile (sequence length -> delta table -> rows) is only exposed once per workgroup.
+    // Virtual block -> (tile, head): consecutive ids go round-robin over the 8 XCDs, each with its own L2; ids are
+    // regrouped so that XCD_GROUP tiles that are neighbours along the query axis -- the tiles that read the same K
+    // and V -- run on one XCD and fetch K / V from HBM once instead of once each.
     const int tiles_x = p.varlen ? p.total / BM + p.B : p.B * ((p.L + BM - 1) / BM);
-    int tile_id, head;
-    {
-        const int n = blockIdx.x, xcd = n & 7, slot = n >> 3;
-        const int v = ((slot / XCD_GROUP) * 8 + xcd) * XCD_GROUP + slot % XCD_GROUP;
-        if (v >= tiles_x * p.H) return;
-        head = v / tiles_x;
-        tile_id = v - head * tiles_x;
-    }
-
-    int b, row0, len;
-    int64_t tok0;
-    if (!tdb_locate_tile(p, BM, tile_id, b, row0, len, tok0)) return;
-
-    const uint16_t* Q = static_cast<const uint16_t*>(p.q) + (p.varlen ? tok0 * p.qs_l : int64_t(b) * p.qs_b) + int64_t(head) * p.qs_h;
-    const uint16_t* K = static_cast<const uint16_t*>(p.k) + (p.varlen ? tok0 * p.ks_l : int64_t(b) * p.ks_b) + int64_t(head) * p.ks_h;
-    const uint16_t* V = static_cast<const uint16_t*>(p.v) + (p.varlen ? tok0 * p.vs_l : int64_t(b) * p.vs_b) + int64_t(head) * p.vs_h;
-    uint16_t* O = static_cast<uint16_t*>(p.o) + (p.varlen ? tok0 * p.os_l : int64_t(b) * p.os_b) + int64_t(head) * p.os_h;
-    const int rows_here = min(BM, (p.varlen ? len : p.L) - row0);   // rows of this tile that exist in memory
-
-    if (row0 >= len) {   // only padded query rows (fixed layout): zeros
-        for (int idx = tid; idx < rows_here * (D / 8); idx += NTHREADS)
-            *reinterpret_cast<u32x4*>(O + int64_t(row0 + (idx >> 3)) * p.os_l + (idx & 7) * 8) = u32x4{0, 0, 0, 0};
-        return;
-    }
-
-    const uint16_t* PK = HAS_C2P ? static_cast<const uint16_t*>(p.pk) + int64_t(head) * p.pks_h : nullptr;
-    const uint16_t* PQ = HAS_P2C ? static_cast<const uint16_t*>(p.pq) + int64_t(head) * p.pqs_h : nullptr;
     const int lut_max = 2 * p.lut_half;
     auto delta_of = [&](int r) { return p.lut[min(max(r + p.lut_half, 0), lut_max)]; };
 
-    // Q^T fragments of query block w: B operand of S^T = K.Q^T (score wave) and of C'^T = K_r'.Q^T (position wave)
-    const int qi = row0 + 32 * w + il;
-    bf16x8 qb[4];
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
-        u32x4 t = {0, 0, 0, 0};
-        if (qi < len) t = *reinterpret_cast<const u32x4*>(Q + int64_t(qi) * p.qs_l + 16 * c + 8 * hh);
-        qb[c] = __builtin_bit_cast(bf16x8, t);
+    struct Tile {
+        int vb, head, b, row0, len;
+        int64_t tok0;
+    };
+    auto tile_index = [&](int vb, int& hd, int& tile_id) {   // false: the virtual block has no tile
+        const int xcd = vb & 7, slot = vb >> 3;
+        const int v = ((slot / XCD_GROUP) * 8 + xcd) * XCD_GROUP + slot % XCD_GROUP;
+        if (vb >= nblocks || v >= tiles_x * p.H) return false;
+        hd = v / tiles_x;
+        tile_id = v - hd * tiles_x;
+        return true;
+    };
+    // Packed launches: every wave keeps the boundaries of the first 64 sequences (one per lane), so that looking a
+    // tile up reads nothing from memory for batches of up to 64 sequences.
+    int cu_lo = 0, cu_hi = 0;
+    if (p.varlen) {
+        cu_lo = p.cu_seqlens[min(l, p.B)];
+        cu_hi = p.cu_seqlens[min(l + 1, p.B)];
     }
+    // tile_id -> (sequence, first row, valid length, first token): same map as tdb_locate_tile, with the packed
+    // boundaries of the first chunk out of registers and the sequence length of sequence pf_b given as pf_len
+    // (read ahead of time by the caller; pf_b = -1: none).
+    auto locate = [&](int tile_id, int pf_b, int pf_len, int& bb, int& r0, int& ln, int64_t& t0) {
+        if (!p.varlen) {
+            const int tiles = (p.L + BM - 1) / BM;
+            bb = tile_id / tiles;
+            r0 = (tile_id - bb * tiles) * BM;
+            const int raw = p.seqlens ? (bb == pf_b ? __builtin_amdgcn_readfirstlane(pf_len) : p.seqlens[bb]) : p.L;
+            ln = min(max(raw, 0), p.L);
+            t0 = 0;
+            return true;
+        }
+        int t = tile_id;
+        for (int b0 = 0; b0 < p.B; b0 += 64) {
+            const int bx = b0 + l;
+            int s0 = 0, n = 0;
+            if (bx < p.B) {
+                s0 = b0 == 0 ? cu_lo : p.cu_seqlens[bx];
+                const int e = b0 == 0 ? cu_hi : p.cu_seqlens[bx + 1];
+                n = e - s0;
+                if (s0 < 0 || n < 0 || e > p.total) n = 0;   // malformed entry: no tiles
+                n = min(n, p.L);
+            }
+            const int nt = (n + BM - 1) / BM;
+            int incl = nt;                                   // inclusive prefix sum over the wave
+#pragma unroll
+            for (int d = 1; d < 64; d <<= 1) {
+                const int up = __shfl_up(incl, d);
+                if (l >= d) incl += up;
+            }
+            const int chunk_tiles = __builtin_amdgcn_readlane(incl, 63);
+            if (t < chunk_tiles) {
+                const unsigned long long owners = __builtin_amdgcn_ballot_w64(incl > t);
+                const int ln_ = __builtin_amdgcn_readfirstlane(__builtin_ctzll(owners));
+                const int before = __builtin_amdgcn_readlane(incl, ln_) - __builtin_amdgcn_readlane(nt, ln_);
+                bb = b0 + ln_;
+                r0 = (t - before) * BM;
+                ln = __builtin_amdgcn_readlane(n, ln_);
+                t0 = __builtin_amdgcn_readlane(s0, ln_);
+                return true;
+            }
+            t -= chunk_tiles;
+        }
+        return false;
+    };
+    // First tile with live query rows among the virtual blocks vb, vb + gridDim.x, ...; vb = -1 if there is none.
+    // Tiles that hold only padded query rows (fixed layout) get their zeros here, from whoever looks them up:
+    // every wave of the workgroup walks the same list, each thread fills its share.
+    auto find_tile = [&](int vb, int pf_b, int pf_len) {
+        Tile t;
+        t.vb = -1;
+        t.head = t.b = t.row0 = t.len = 0;
+        t.tok0 = 0;
+        for (; vb < nblocks; vb += gridDim.x) {
+            int hd, tile_id;
+            if (!tile_index(vb, hd, tile_id)) continue;
+            int bb, r0, ln;
+            int64_t t0;
+            if (!locate(tile_id, pf_b, pf_len, bb, r0, ln, t0)) continue;
+            if (r0 >= ln) {
+                uint16_t* Oz = static_cast<uint16_t*>(p.o) + (p.varlen ? t0 * p.os_l : int64_t(bb) * p.os_b) + int64_t(hd) * p.os_h;
+                const int rows = min(BM, (p.varlen ? ln : p.L) - r0);
+                for (int idx = tid; idx < rows * (D / 8); idx += NTHREADS)
+                    *reinterpret_cast<u32x4*>(Oz + int64_t(r0 + (idx >> 3)) * p.os_l + (idx & 7) * 8) = u32x4{0, 0, 0, 0};
+                continue;
+            }
+            t.vb = vb;
+            t.head = hd;
+            t.b = bb;
+            t.row0 = r0;
+            t.len = ln;
+            t.tok0 = t0;
+            break;
+        }
+        return t;
+    };
+    // Sequence length of the tile of virtual block vb, requested ahead of its lookup (fixed layout).  It is read
+    // through the vector memory path on purpose: a scalar read would be waited for at the next workgroup barrier
+    // (LDS and scalar memory share a counter), a vector read is only waited for where its value is used.
+    auto length_ahead = [&](int vb, int& pf_b, int& pf_len) {
+        pf_b = -1;
+        pf_len = 0;
+        int hd, tile_id;
+        if (!p.varlen && p.seqlens && tile_index(vb, hd, tile_id)) {
+            pf_b = tile_id / ((p.L + BM - 1) / BM);
+            int idx = pf_b;
+            asm volatile("" : "+v"(idx));
+            pf_len = p.seqlens[idx];
+        }
+    };
+    auto k_of = [&](const Tile& t) {
+        return static_cast<const uint16_t*>(p.k) + (p.varlen ? t.tok0 * p.ks_l : int64_t(t.b) * p.ks_b) + int64_t(t.head) * p.ks_h;
+    };
+    auto pk_of = [&](const Tile& t) { return HAS_C2P ? static_cast<const uint16_t*>(p.pk) + int64_t(t.head) * p.pks_h : nullptr; };
+    auto pq_of = [&](const Tile& t) { return HAS_P2C ? static_cast<const uint16_t*>(p.pq) + int64_t(t.head) * p.pqs_h : nullptr; };
 
-    // ---- pipeline ----------------------------------------------------------------------------------------------
+    Tile cur = find_tile(blockIdx.x, -1, 0);
+    if (cur.vb < 0) return;
+
+    // ---- pipeline of one tile -----------------------------------------------------------------------------------
     // Key step s covers keys 64s .. 64s+63 and needs relative positions B_s .. B_s+190, B_s = row0 - 64s - 63.
     // The rows K_r[delta(r)] / Q_r[delta(r)] of that window live in a 192-row ring: going to the next step the
     // window slides down by 64, so only its 64 lowest positions are fetched and they overwrite the 64 highest
     // of the previous step.  Window row x of step s sits in ring slot (x + off_s) mod 192, off_s = (128*s) mod 192.
     //
-    // Each step has two halves separated by workgroup barriers, arranged so that in either half one role is on
-    // the LDS and the other on the matrix cores:
+    // A tile opens with three barriers (first stage in LDS; position products of step 0 in the scratch; window of
+    // step 1 complete).  Then each step has two halves separated by workgroup barriers, arranged so that in either
+    // half one role is on the LDS and the other on the matrix cores:
     //   A  score waves read this step's position terms out of the C'/P' scratch into their score accumulators;
     //      position waves hand register-prefetched global data to LDS (keys of step s+2, values of step s, 64 window
     //      rows of step s+2) and run the 24 position MFMAs of step s+1 on fragments they already hold;
     //   B  score waves: S^T(s), softmax(s), P.V(s), and they pick up the K fragments of step s+1;
     //      position waves: results of step s+1 into the now free scratch, global fetches for the next half A,
     //      LDS fragments of step s+2.
-    const int nsteps = (len + BN - 1) / BN;
-    const int nfull = len / BN;           // steps that need no key mask
+    // Both roles pass 3 + 2*nsteps barriers per tile and walk the same tile list.
     const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     auto prev_off = [](int o) { return o >= BN ? o - BN : o + WIN - BN; };   // ring offset of the following step
 
-    // prologue, all 512 threads: keys of steps 0 and 1 and the whole window of step 0 to LDS
+    // state of the current tile, rebound when the workgroup moves on
+    int row0 = 0, len = 0, nsteps = 0, nfull = 0, rows_here = 0;
+    const uint16_t *Q = nullptr, *K = nullptr, *V = nullptr, *PK = nullptr, *PQ = nullptr;
+    uint16_t* O = nullptr;
+    auto bind = [&](const Tile& t) {
+        row0 = t.row0;
+        len = t.len;
+        nsteps = (len + BN - 1) / BN;
+        nfull = len / BN;                 // steps that need no key mask
+        rows_here = min(BM, (p.varlen ? len : p.L) - row0);   // rows of this tile that exist in memory
+        Q = static_cast<const uint16_t*>(p.q) + (p.varlen ? t.tok0 * p.qs_l : int64_t(t.b) * p.qs_b) + int64_t(t.head) * p.qs_h;
+        K = k_of(t);
+        V = static_cast<const uint16_t*>(p.v) + (p.varlen ? t.tok0 * p.vs_l : int64_t(t.b) * p.vs_b) + int64_t(t.head) * p.vs_h;
+        O = static_cast<uint16_t*>(p.o) + (p.varlen ? t.tok0 * p.os_l : int64_t(t.b) * p.os_b) + int64_t(t.head) * p.os_h;
+        PK = pk_of(t);
+        PQ = pq_of(t);
+    };
+    bind(cur);
+
+    // Q^T fragments of query block w: B operand of S^T = K.Q^T (score wave) and of C'^T = K_r'.Q^T (position wave)
+    bf16x8 qb[4];
+    auto load_q = [&](bf16x8 (&dst)[4], const Tile& t) {
+        const uint16_t* Qt = static_cast<const uint16_t*>(p.q) + (p.varlen ? t.tok0 * p.qs_l : int64_t(t.b) * p.qs_b) + int64_t(t.head) * p.qs_h;
+        const int qrow = t.row0 + 32 * w + il;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            u32x4 x = {0, 0, 0, 0};
+            if (t.vb >= 0 && qrow < t.len) x = *reinterpret_cast<const u32x4*>(Qt + int64_t(qrow) * p.qs_l + 16 * c + 8 * hh);
+            dst[c] = __builtin_bit_cast(bf16x8, x);
+        }
+    };
+    load_q(qb, cur);
+
+    // First tile of the workgroup: nothing was requested ahead, so all 512 threads share its first LDS stage (keys of
+    // steps 0 and 1, the whole window of step 0: 8 chunks of 16 B per thread) and the chain of dependent reads
+    // (delta table -> rows) is as short as it can be.  Later tiles are staged by the position waves alone, with
+    // reads issued a key step ahead.
+    int dl_cold[3][2] = {{0, 0}, {0, 0}, {0, 0}};   // position waves: delta of the new window rows of steps 1 to 3
     {
-        const int row = tid >> 3, ch = tid & 7;              // rows 0..63
-        *reinterpret_cast<u32x4*>(&sm.k[0][row * RS + ch * 8]) =
-            *reinterpret_cast<const u32x4*>(K + int64_t(min(row, len - 1)) * p.ks_l + ch * 8);
-        *reinterpret_cast<u32x4*>(&sm.k[1][row * RS + ch * 8]) =
-            *reinterpret_cast<const u32x4*>(K + int64_t(min(BN + row, len - 1)) * p.ks_l + ch * 8);
+        const int row = tid >> 3, ch = tid & 7;     // rows 0..63
+        int dl[WIN / 64] = {0, 0, 0};
         if (HAS_POS) {
 #pragma unroll
-            for (int n = 0; n < WIN / 64; ++n) {
-                const int x = row + 64 * n;
-                const int dl = delta_of(row0 - (BN - 1) + x);
-                if (HAS_C2P)
-                    *reinterpret_cast<u32x4*>(&sm.kr[x * RS + ch * 8]) = *reinterpret_cast<const u32x4*>(PK + int64_t(dl) * p.pks_r + ch * 8);
-                if (HAS_P2C)
-                    *reinterpret_cast<u32x4*>(&sm.qr[x * RS + ch * 8]) = *reinterpret_cast<const u32x4*>(PQ + int64_t(dl) * p.pqs_r + ch * 8);
+            for (int n = 0; n < WIN / 64; ++n) dl[n] = delta_of(row0 - (BN - 1) + row + 64 * n);
+            if (!score_role) {
+#pragma unroll
+                for (int s1 = 0; s1 < 3; ++s1)
+#pragma unroll
+                    for (int n = 0; n < 2; ++n)
+                        dl_cold[s1][n] = delta_of(row0 - BN * (s1 + 1) - (BN - 1) + ((tid - 256) >> 3) + 32 * n);
             }
         }
+        const u32x4 k0 = *reinterpret_cast<const u32x4*>(K + int64_t(min(row, len - 1)) * p.ks_l + ch * 8);
+        const u32x4 k1 = *reinterpret_cast<const u32x4*>(K + int64_t(min(BN + row, len - 1)) * p.ks_l + ch * 8);
+        u32x4 wk[WIN / 64], wq[WIN / 64];
+#pragma unroll
+        for (int n = 0; n < WIN / 64; ++n) {
+            if (HAS_C2P) wk[n] = *reinterpret_cast<const u32x4*>(PK + int64_t(dl[n]) * p.pks_r + ch * 8);
+            if (HAS_P2C) wq[n] = *reinterpret_cast<const u32x4*>(PQ + int64_t(dl[n]) * p.pqs_r + ch * 8);
+        }
+        *reinterpret_cast<u32x4*>(&sm.k[0][row * RS + ch * 8]) = k0;
+        *reinterpret_cast<u32x4*>(&sm.k[1][row * RS + ch * 8]) = k1;
+#pragma unroll
+        for (int n = 0; n < WIN / 64; ++n) {
+            if (HAS_C2P) *reinterpret_cast<u32x4*>(&sm.kr[(row + 64 * n) * RS + ch * 8]) = wk[n];
+            if (HAS_P2C) *reinterpret_cast<u32x4*>(&sm.qr[(row + 64 * n) * RS + ch * 8]) = wq[n];
+        }
     }
-    __syncthreads();
 
     if (!score_role) {
         // ================================================= position waves ==========================================
         const int stid = tid - 256;
-        const int srow = stid >> 3, sch = stid & 7;          // this thread stages rows srow, srow+32 (chunk sch)
+        const int srow = stid >> 3, sch = stid & 7;          // this thread stages rows srow + 32n (chunk sch)
         // global -> registers through buffer loads.  The buffer of a step starts at its first row and ends with the
         // last row of the sequence, so rows past the end come back as zeros (hardware range check) with no lane
         // predicated off, and the per-load address arithmetic is scalar.
-        const int ks_b = int(p.ks_l) * 2, vs_b = int(p.vs_l) * 2, pks_b = int(p.pks_r) * 2, pqs_b = int(p.pqs_r) * 2;
-        int kvoff[2], vvoff[2];
-#pragma unroll
-        for (int n = 0; n < 2; ++n) {
-            kvoff[n] = (srow + 32 * n) * ks_b + sch * 16;
-            vvoff[n] = (srow + 32 * n) * vs_b + sch * 16;
-        }
-        const __amdgpu_buffer_rsrc_t pk_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-            const_cast<uint16_t*>(HAS_C2P ? PK : K), 0, HAS_C2P ? (2 * p.span - 1) * pks_b + 128 : 0, RSRC_FLAGS);
-        const __amdgpu_buffer_rsrc_t pq_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-            const_cast<uint16_t*>(HAS_P2C ? PQ : K), 0, HAS_P2C ? (2 * p.span - 1) * pqs_b + 128 : 0, RSRC_FLAGS);
-        u32x4 pre_k[2], pre_v[2], pre_kr[2], pre_qr[2];
+        const int pks_b = int(p.pks_r) * 2, pqs_b = int(p.pqs_r) * 2;
+        __amdgpu_buffer_rsrc_t pk_rsrc, pq_rsrc;
+        auto bind_tables = [&]() {
+            pk_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(HAS_C2P ? PK : K), 0,
+                                                        HAS_C2P ? (2 * p.span - 1) * pks_b + 128 : 0, RSRC_FLAGS);
+            pq_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(HAS_P2C ? PQ : K), 0,
+                                                        HAS_P2C ? (2 * p.span - 1) * pqs_b + 128 : 0, RSRC_FLAGS);
+        };
+        u32x4 pre_kr[2], pre_qr[2];
         int dl_next[2] = {0, 0};
-        auto fetch = [&](int sk, int sv) {     // key rows of step sk, value rows of step sv, new window rows (dl_next)
-            const int kleft = len - BN * sk, vleft = len - BN * sv;
-            const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-                const_cast<uint16_t*>(K) + int64_t(BN * sk) * p.ks_l, 0, kleft > 0 ? (kleft - 1) * ks_b + 128 : 0, RSRC_FLAGS);
-            const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-                const_cast<uint16_t*>(V) + int64_t(BN * sv) * p.vs_l, 0, vleft > 0 ? (vleft - 1) * vs_b + 128 : 0, RSRC_FLAGS);
+        auto fetch = [&]() {                   // the 64 new window rows of a step (dl_next)
 #pragma unroll
             for (int n = 0; n < 2; ++n) {
-                pre_k[n] = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, kvoff[n], 0, 0);
-                pre_v[n] = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, vvoff[n], 0, 0);
                 if (HAS_C2P) pre_kr[n] = __builtin_amdgcn_raw_buffer_load_b128(pk_rsrc, dl_next[n] * pks_b + sch * 16, 0, 0);
                 if (HAS_P2C) pre_qr[n] = __builtin_amdgcn_raw_buffer_load_b128(pq_rsrc, dl_next[n] * pqs_b + sch * 16, 0, 0);
             }
@@ -252,12 +412,10 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
                 for (int n = 0; n < 2; ++n) dl_next[n] = delta_of(row0 - BN * s - (BN - 1) + srow + 32 * n);
             }
         };
-        auto store = [&](int o, int kbuf) {    // registers -> LDS: keys into k[kbuf], window rows at ring offset o
+        auto store = [&](int o) {              // registers -> LDS: window rows at ring offset o
 #pragma unroll
             for (int n = 0; n < 2; ++n) {
                 const int r = srow + 32 * n;
-                *reinterpret_cast<u32x4*>(&sm.k[kbuf][r * RS + sch * 8]) = pre_k[n];
-                *reinterpret_cast<u32x4*>(&sm.v[r * RS + sch * 8]) = pre_v[n];
                 if (HAS_C2P) *reinterpret_cast<u32x4*>(&sm.kr[(o + r) * RS + sch * 8]) = pre_kr[n];
                 if (HAS_P2C) *reinterpret_cast<u32x4*>(&sm.qr[(o + r) * RS + sch * 8]) = pre_qr[n];
             }
@@ -339,67 +497,205 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
             }
         };
 
-        // prologue: products of step 0; window rows of step 1 (they overwrite rows step 0 is done with);
-        // fragments of step 1; prefetch for half A of step 0
-        const int off1 = prev_off(0);
-        fetch_delta(1);
-        load_frags(0, 0);
-        products();
-        put_results();
-        fetch(2, 0);                      // pre_k: keys of step 2 (unused rows of step 1), pre_v: values of step 0
-        phase_barrier();                  // every position wave has its fragments of step 0
-        if (HAS_POS) {
+        // First LDS stage of a tile: keys of steps 0 and 1 and the whole window of step 0 (192 rows of either
+        // table), 16 chunks of 16 B per thread.  The delta values come first (dl_win for the window, dl_step for
+        // the 64 new rows of steps 1 to 3), the row reads depend on them.
+        int dl_win[WIN / 32], dl_step[3][2];
+        u32x4 st_k[4], st_wk[WIN / 32], st_wq[WIN / 32];
+        bf16x8 qb_next[4];
+        // (Both readers assign every register also when there is no next tile: a conditional assignment would keep the
+        // previous tile's values alive across the whole tile body.)
+        auto read_deltas = [&](const Tile& t) {
 #pragma unroll
-            for (int n = 0; n < 2; ++n) {
-                const int r = srow + 32 * n;
-                if (HAS_C2P) *reinterpret_cast<u32x4*>(&sm.kr[(off1 + r) * RS + sch * 8]) = pre_kr[n];
-                if (HAS_P2C) *reinterpret_cast<u32x4*>(&sm.qr[(off1 + r) * RS + sch * 8]) = pre_qr[n];
+            for (int n = 0; n < WIN / 32; ++n) dl_win[n] = 0;
+#pragma unroll
+            for (int s1 = 0; s1 < 3; ++s1) dl_step[s1][0] = dl_step[s1][1] = 0;
+            if (HAS_POS && t.vb >= 0) {
+                int sr = srow;            // opaque: keeps a dozen precomputed row offsets out of long-lived registers
+                asm volatile("" : "+v"(sr));
+#pragma unroll
+                for (int n = 0; n < WIN / 32; ++n) dl_win[n] = delta_of(t.row0 - (BN - 1) + sr + 32 * n);
+#pragma unroll
+                for (int s1 = 0; s1 < 3; ++s1)
+#pragma unroll
+                    for (int n = 0; n < 2; ++n) dl_step[s1][n] = delta_of(t.row0 - BN * (s1 + 1) - (BN - 1) + sr + 32 * n);
             }
+        };
+        auto read_stage = [&](const Tile& t) {
+            const uint16_t *Kt = k_of(t), *PKt = pk_of(t), *PQt = pq_of(t);
+            const u32x4 none = {0, 0, 0, 0};
+#pragma unroll
+            for (int n = 0; n < 4; ++n) st_k[n] = none;
+#pragma unroll
+            for (int n = 0; n < WIN / 32; ++n) st_wk[n] = st_wq[n] = none;
+            if (t.vb >= 0) {
+#pragma unroll
+                for (int n = 0; n < 4; ++n)
+                    st_k[n] = *reinterpret_cast<const u32x4*>(Kt + int64_t(min(srow + 32 * n, t.len - 1)) * p.ks_l + sch * 8);
+#pragma unroll
+                for (int n = 0; n < WIN / 32; ++n) {
+                    if (HAS_C2P) st_wk[n] = *reinterpret_cast<const u32x4*>(PKt + int64_t(dl_win[n]) * p.pks_r + sch * 8);
+                    if (HAS_P2C) st_wq[n] = *reinterpret_cast<const u32x4*>(PQt + int64_t(dl_win[n]) * p.pqs_r + sch * 8);
+                }
+            }
+        };
+        auto write_stage = [&]() {
+#pragma unroll
+            for (int n = 0; n < 4; ++n)
+                *reinterpret_cast<u32x4*>(&sm.k[n >> 1][(srow + 32 * (n & 1)) * RS + sch * 8]) = st_k[n];
+#pragma unroll
+            for (int n = 0; n < WIN / 32; ++n) {
+                if (HAS_C2P) *reinterpret_cast<u32x4*>(&sm.kr[(srow + 32 * n) * RS + sch * 8]) = st_wk[n];
+                if (HAS_P2C) *reinterpret_cast<u32x4*>(&sm.qr[(srow + 32 * n) * RS + sch * 8]) = st_wq[n];
+            }
+        };
+
+#pragma unroll
+        for (int s1 = 0; s1 < 3; ++s1) {
+            dl_step[s1][0] = dl_cold[s1][0];
+            dl_step[s1][1] = dl_cold[s1][1];
         }
-        fetch_delta(2);
-        phase_barrier();                  // window of step 1 complete
-        load_frags(off1, 1);
-        fetch(2, 0);                      // keys of step 2, values of step 0, window rows of step 2
-        fetch_delta(3);
-        int off2 = prev_off(off1);        // ring offset of step s+2
-        for (int s = 0; s < nsteps; ++s) {
-            phase_barrier();              // scratch of step s complete
-            products();                   // of step s+1, into registers; issued first: the wait for the
-            __builtin_amdgcn_sched_barrier(0);  // prefetched global data then passes under the MFMAs
-            store(off2, s & 1);           // keys of step s+2, values of step s, new window rows of step s+2
-            phase_barrier();              // score waves are done with the scratch; the staged tiles are visible
-            put_results();                // of step s+1 (harmless left-over work in the last step)
-            fetch(s + 3, s + 1);
-            fetch_delta(s + 4);
-            load_frags(off2, s & 1);      // of step s+2
-            off2 = prev_off(off2);
+        TDB_T_DECL
+        while (true) {
+            TDB_PRESET;
+            bind_tables();
+            // The tile after this one is looked up here, where the wait for its sequence length falls into the
+            // wait for the score waves; its delta values are read in the last step but one (when the fragment and
+            // result registers are no longer needed), its first stage during the last step.
+            int pf_b, pf_len;             // asked for here, used by the lookup after the opening barriers
+            length_ahead(cur.vb + gridDim.x, pf_b, pf_len);
+            phase_barrier();              // first stage of the tile is in LDS
+            TDB_PSTAMP(1);
+            // products of step 0; window rows of step 1 (they overwrite rows step 0 is done with); fragments of
+            // step 1; prefetch for half A of step 0
+            const int off1 = prev_off(0);
+            dl_next[0] = dl_step[0][0];
+            dl_next[1] = dl_step[0][1];
+            fetch();                      // window rows of step 1; they arrive under the products of step 0
+            load_frags(0, 0);
+            products();
+            put_results();
+            TDB_PSTAMP(2);
+            phase_barrier();              // every position wave has its fragments of step 0
+            TDB_PSTAMP(3);
+            store(off1);
+            dl_next[0] = dl_step[1][0];
+            dl_next[1] = dl_step[1][1];
+            fetch();                      // window rows of step 2
+            dl_next[0] = dl_step[2][0];
+            dl_next[1] = dl_step[2][1];
+            TDB_PSTAMP(4);
+            phase_barrier();              // window of step 1 complete
+            TDB_PSTAMP(5);
+            load_frags(off1, 1);
+            TDB_PSTAMP(6);
+            // The tile after this one: its delta values are read in the last step but one (when the fragment and
+            // result registers are no longer needed), its first stage during the last step.
+            const Tile nxt = find_tile(cur.vb + gridDim.x, pf_b, pf_len);
+            TDB_PSTAMP(7);
+
+            int off2 = prev_off(off1);    // ring offset of step s+2
+            auto pos_step = [&](int s, auto tail_tag) {
+                constexpr bool TAIL = decltype(tail_tag)::value;   // step nsteps-2: no step s+2 to prepare
+                phase_barrier();          // scratch of step s complete
+                TDB_STAMP(0);
+                products();               // of step s+1, into registers; issued first: the wait for the
+                __builtin_amdgcn_sched_barrier(0);  // prefetched global data then passes under the MFMAs
+                store(off2);              // new window rows of step s+2
+                if (!TAIL) {
+                    fetch();              // window rows of step s+3: a full step ahead of their store
+                    fetch_delta(s + 4);
+                }
+                TDB_STAMP(1);
+                phase_barrier();          // score waves are done with the scratch; the staged tiles are visible
+                TDB_STAMP(2);
+                put_results();            // of step s+1
+                if (!TAIL) load_frags(off2, s & 1);  // of step s+2
+                off2 = prev_off(off2);
+                TDB_STAMP(3);
+            };
+            if (nsteps >= 2) {
+                for (int s = 0; s + 2 < nsteps; ++s) pos_step(s, std::false_type{});
+                pos_step(nsteps - 2, std::true_type{});
+            }
+            read_deltas(nxt);
+            // last key step: nothing left to prepare for this tile; the first stage of the next tile is requested
+            phase_barrier();
+            TDB_STAMP(0);
+            read_stage(nxt);
+            load_q(qb_next, nxt);
+            TDB_STAMP(1);
+            phase_barrier();
+            TDB_STAMP(2);
+            if (nxt.vb < 0) break;
+            write_stage();                // (the score waves are still in half B of the last step: they read only V)
+            TDB_PSTAMP(0);
+            cur = nxt;
+            bind(cur);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) qb[c] = qb_next[c];
         }
+        TDB_T_FLUSH(6);
+        TDB_P_FLUSH;
         return;
     }
 
     // ===================================================== score waves ============================================
-    f32x16 o_acc[2] = {zero16, zero16};
-    float m_run = -INFINITY, l_run = 0.f;
     const float c_exp = p.scale * 1.4426950408889634f;   // softmax in base 2
     const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
+    f32x16 o_acc[2];
+    float m_run, l_run;
 
-    bf16x8 kf[2][4], kf2[2][4];           // K fragments: A operand of S^T = K.Q^T; two sets that swap roles
-    auto load_kf = [&](bf16x8 (&dst)[2][4], int kbuf) {
+    bf16x8 kf[2][4];                      // K fragments: A operand of S^T = K.Q^T
+    auto load_kf = [&](int kbuf) {
 #pragma unroll
         for (int jt = 0; jt < 2; ++jt)
 #pragma unroll
-            for (int c = 0; c < 4; ++c) dst[jt][c] = lds_frag(sm.k[kbuf], 32 * jt + il, 16 * c + 8 * hh);
+            for (int c = 0; c < 4; ++c) kf[jt][c] = lds_frag(sm.k[kbuf], 32 * jt + il, 16 * c + 8 * hh);
     };
-    load_kf(kf, 0);
-    phase_barrier();                      // the two prologue barriers of the position waves
-    phase_barrier();
+    // Keys and values travel global -> registers -> LDS through the score waves: thread tid stages chunk sch of rows
+    // srow and srow + 32 of a 64-row step.  Buffer loads: the buffer of a step starts at its first row and ends with
+    // the last row of the sequence, so rows past the end come back as zeros (hardware range check) with no lane
+    // predicated off, and the per-load address arithmetic is scalar.
+    const int srow = tid >> 3, sch = tid & 7;
+    const int ks_b = int(p.ks_l) * 2, vs_b = int(p.vs_l) * 2;
+    int kvoff[2], vvoff[2];
+#pragma unroll
+    for (int n = 0; n < 2; ++n) {
+        kvoff[n] = (srow + 32 * n) * ks_b + sch * 16;
+        vvoff[n] = (srow + 32 * n) * vs_b + sch * 16;
+    }
+    u32x4 pre_k[2], pre_v[2];
+    auto fetch_kv = [&](int sk, int sv) {  // key rows of step sk, value rows of step sv
+        const int kleft = len - BN * sk, vleft = len - BN * sv;
+        const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<uint16_t*>(K) + int64_t(BN * sk) * p.ks_l, 0, kleft > 0 ? (kleft - 1) * ks_b + 128 : 0, RSRC_FLAGS);
+        const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<uint16_t*>(V) + int64_t(BN * sv) * p.vs_l, 0, vleft > 0 ? (vleft - 1) * vs_b + 128 : 0, RSRC_FLAGS);
+#pragma unroll
+        for (int n = 0; n < 2; ++n) {
+            pre_k[n] = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, kvoff[n], 0, 0);
+            pre_v[n] = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, vvoff[n], 0, 0);
+        }
+    };
+    auto store_kv = [&](int kbuf) {
+#pragma unroll
+        for (int n = 0; n < 2; ++n) {
+            *reinterpret_cast<u32x4*>(&sm.k[kbuf][(srow + 32 * n) * RS + sch * 8]) = pre_k[n];
+            *reinterpret_cast<u32x4*>(&sm.v[(srow + 32 * n) * RS + sch * 8]) = pre_v[n];
+        }
+    };
+    TDB_T_DECL
     // One key step.  MASKED: the step reaches past the end of the sequence (only the last step can).
-    auto key_step = [&](int s, const bf16x8 (&kc)[2][4], bf16x8 (&kn)[2][4], auto masked_tag) {
+    auto key_step = [&](int s, auto masked_tag) {
         constexpr bool MASKED = decltype(masked_tag)::value;
         phase_barrier();                  // scratch of step s complete
+        TDB_STAMP(0);
 
-        // ---- half A: position terms of step s out of the scratch.  Element (jj, i) of the score tile takes
+        // ---- half A: keys of step s+2 and values of step s go to LDS (prefetched registers, nothing waits);
+        //      position terms of step s out of the scratch.  Element (jj, i) of the score tile takes
         //      C'[i][i-jj+63] (fp32, straight into the accumulator) and P'[jj][32w+i-jj+63] (bf16) ----------------
+        store_kv(s & 1);
         f32x16 s_acc[2];
         if (HAS_C2P) {
             // float index of element e of key tile jt:  il*CS + il + 63 - 4*hh - jc,  jc = 32*jt + 8*(e>>2) + (e&3) <= 59
@@ -433,14 +729,17 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
                 for (int e = 0; e < 16; ++e)   // bf16 pair (value, 0) . (1, 1) + acc
                     s_acc[jt][e] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, g[jt][e]), ones, s_acc[jt][e], false);
         }
+        TDB_STAMP(1);
         phase_barrier();                  // scratch is free again; keys of step s+1 and values of step s are staged
+        TDB_STAMP(2);
 
         // ---- half B ---------------------------------------------------------------------------------------------
 #pragma unroll
         for (int c = 0; c < 4; ++c)
 #pragma unroll
-            for (int jt = 0; jt < 2; ++jt) s_acc[jt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kc[jt][c], qb[c], s_acc[jt], 0, 0, 0);
-        load_kf(kn, (s + 1) & 1);         // K fragments of step s+1
+            for (int jt = 0; jt < 2; ++jt) s_acc[jt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[jt][c], qb[c], s_acc[jt], 0, 0, 0);
+        load_kf((s + 1) & 1);             // K fragments of step s+1 (the MFMAs above have read this step's)
+        fetch_kv(s + 3, s + 1);           // for the next half A
         // V^T fragments through the transposing LDS read: the lane provides the address of 4 dims of one key
         bf16x8 vf[2][2][2];               // [key tile][16-key chunk][dim tile]
         {
@@ -510,35 +809,95 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
                     o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[jt][c][dt], pb, o_acc[dt], 0, 0, 0);
             }
         l_run += psum;
+        TDB_STAMP(3);
     };
 
-    // steps run in pairs so that the two sets of K fragment registers just swap roles
-    int s = 0;
-    for (; s + 1 < nfull; s += 2) {
-        key_step(s, kf, kf2, std::false_type{});
-        key_step(s + 1, kf2, kf, std::false_type{});
-    }
-    if (s < nfull) {
-        key_step(s, kf, kf2, std::false_type{});
-        if (nfull < nsteps) key_step(nfull, kf2, kf, std::true_type{});
-    } else if (nfull < nsteps) {
-        key_step(nfull, kf, kf2, std::true_type{});
-    }
-
-    // ---- epilogue: normalise and store O[i][d]; lane holds d = 32*dt + 8*a + 4*hh + 0..3 of query row il ------
-    const float l_tot = l_run + __shfl_xor(l_run, 32);
-    const float inv = 1.f / l_tot;
-    if (qi < row0 + rows_here) {
+    // Opening of a tile, after its first barrier (first stage in LDS).  Everything that reads global memory is
+    // requested here and waited for much later: keys of step 2 / values of step 0 (stored in half A of step 0), the
+    // sequence length and Q fragments of the tile after this one.  The output rows of the previous tile are written
+    // last: stores count on the same in-order counter as loads, so a wait for any load issued after them would
+    // also wait for them.
+    int pf_b, pf_len;                     // sequence length of the next tile, asked for one tile ahead of its lookup
+    length_ahead(cur.vb + gridDim.x, pf_b, pf_len);
+    Tile nxt;
+    bf16x8 qb_next[4];
+    u32x2 o_out[2][4];                    // packed output rows of the tile just finished
+    uint16_t* o_ptr = nullptr;
+    bool o_write = false;
+    auto open_tile = [&]() {
+        TDB_PRESET;
+        load_kf(0);
+        TDB_PSTAMP(0);
+        nxt = find_tile(cur.vb + gridDim.x, pf_b, pf_len);
+        TDB_PSTAMP(1);
+        length_ahead(nxt.vb >= 0 ? nxt.vb + gridDim.x : nblocks, pf_b, pf_len);
+        fetch_kv(2, 0);
+        load_q(qb_next, nxt);
+        TDB_PSTAMP(2);
+        if (o_write) {
+#pragma unroll
+            for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+                for (int a = 0; a < 4; ++a) *reinterpret_cast<u32x2*>(o_ptr + 32 * dt + 8 * a) = o_out[dt][a];
+        }
+        TDB_PSTAMP(3);
+        phase_barrier();                  // the two opening barriers of the position waves
+        TDB_PSTAMP(4);
+        phase_barrier();
+        TDB_PSTAMP(5);
+    };
+    // epilogue of a tile: normalised output rows, packed; lane holds d = 32*dt + 8*a + 4*hh + 0..3 of query row il
+    auto close_tile = [&]() {
+        const int qi = row0 + 32 * w + il;
+        const float l_tot = l_run + __shfl_xor(l_run, 32);
+        const float inv = 1.f / l_tot;
         const bool live = qi < len;
+        o_write = qi < row0 + rows_here;
+        o_ptr = O + int64_t(qi) * p.os_l + 4 * hh;
 #pragma unroll
         for (int dt = 0; dt < 2; ++dt)
 #pragma unroll
             for (int a = 0; a < 4; ++a) {
                 u32x2 r = {0, 0};
                 if (live) r = pack4(o_acc[dt][4 * a] * inv, o_acc[dt][4 * a + 1] * inv, o_acc[dt][4 * a + 2] * inv, o_acc[dt][4 * a + 3] * inv);
-                *reinterpret_cast<u32x2*>(O + int64_t(qi) * p.os_l + 32 * dt + 8 * a + 4 * hh) = r;
+                o_out[dt][a] = r;
             }
+    };
+
+    phase_barrier();                      // first stage of the first tile is in LDS
+    open_tile();
+    while (true) {
+        o_acc[0] = zero16;
+        o_acc[1] = zero16;
+        m_run = -INFINITY;
+        l_run = 0.f;
+        for (int s = 0; s < nfull; ++s) key_step(s, std::false_type{});
+        if (nfull < nsteps) key_step(nfull, std::true_type{});
+
+        // The position waves have put the first stage of the next tile into LDS in the meantime and go on to its
+        // first position products; this tile is closed under those.
+        TDB_PRESET;
+        if (nxt.vb >= 0) phase_barrier();
+        TDB_PSTAMP(6);
+        close_tile();
+        TDB_PSTAMP(7);
+        TDB_STAMP(5);
+        if (nxt.vb < 0) break;
+        cur = nxt;
+        bind(cur);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) qb[c] = qb_next[c];
+        open_tile();
     }
+    if (o_write) {
+#pragma unroll
+        for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+            for (int a = 0; a < 4; ++a) *reinterpret_cast<u32x2*>(o_ptr + 32 * dt + 8 * a) = o_out[dt][a];
+    }
+    TDB_T_FLUSH(0);
+    TDB_P_FLUSH;
+    TDB_TRACE_EXIT;
 }
 
 }  // namespace
@@ -558,7 +917,21 @@ bool tdb_mfma_supported(const TdbKernelParams& p, int dtype) {
 hipError_t tdb_launch_mfma(const TdbKernelParams& p, int, hipStream_t stream) {
     const int64_t tiles = int64_t(p.varlen ? p.total / BM + p.B : p.B * ((p.L + BM - 1) / BM)) * p.H;
     const int64_t round = 8 * XCD_GROUP;                 // the id regrouping is a bijection on multiples of this
-    const dim3 grid(unsigned((tiles + round - 1) / round * round)), block(NTHREADS);
+    const int nblocks = int((tiles + round - 1) / round * round);
+    // persistent workgroups: one per CU, in multiples of the 8 XCDs the ids are dealt over
+    static int cus_of[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
+    if (cus_of[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 8) n = 8;
+        cus_of[dev] = n / 8 * 8;
+    }
+    // Fixed layout: persistent workgroups, one per CU (tiles cost the same, a static deal is balanced).  Packed:
+    // tiles differ in length by up to 8x, so every tile gets its own workgroup and the hardware dispatcher hands
+    // them to CUs as they free up.
+    const int persistent = nblocks < cus_of[dev] ? nblocks : cus_of[dev];
+    const dim3 grid(unsigned(p.varlen ? nblocks : persistent)), block(NTHREADS);
     const size_t smem = sizeof(Smem);
     const bool c2p = p.pk != nullptr, p2c = p.pq != nullptr;
 #define TDB_LAUNCH(A, B)                                                                                        \
@@ -569,7 +942,7 @@ hipError_t tdb_launch_mfma(const TdbKernelParams& p, int, hipStream_t stream) {
                                 hipFuncAttributeMaxDynamicSharedMemorySize, int(smem));                         \
             attr_set = true;                                                                                    \
         }                                                                                                       \
-        hipLaunchKernelGGL((attn_mfma_kernel<A, B>), grid, block, smem, stream, p);                             \
+        hipLaunchKernelGGL((attn_mfma_kernel<A, B>), grid, block, smem, stream, p, nblocks);                        \
     } while (0)
     if (c2p && p2c) TDB_LAUNCH(true, true);
     else if (c2p) TDB_LAUNCH(true, false);
@@ -578,3 +951,4 @@ hipError_t tdb_launch_mfma(const TdbKernelParams& p, int, hipStream_t stream) {
 #undef TDB_LAUNCH
     return hipGetLastError();
 }
+
