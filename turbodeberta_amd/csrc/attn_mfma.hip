@@ -90,6 +90,12 @@ __device__ __forceinline__ float2 lds_read2_f32(uint32_t addr) {
     asm volatile("ds_read2_b32 %0, %1 offset0:%2 offset1:%3" : "=v"(r) : "v"(addr), "n"(OFF0), "n"(OFF1) : "memory");
     return r;
 }
+template <int OFF0, int OFF1>   // the same, as raw dwords
+__device__ __forceinline__ u32x2 lds_read2_u32(uint32_t addr) {
+    u32x2 r;
+    asm volatile("ds_read2_b32 %0, %1 offset0:%2 offset1:%3" : "=v"(r) : "v"(addr), "n"(OFF0), "n"(OFF1) : "memory");
+    return r;
+}
 template <int OFF>              // one zero-extended 16-bit value at byte offset OFF
 __device__ __forceinline__ uint32_t lds_read_u16(uint32_t addr) {
     uint32_t r;
@@ -713,12 +719,26 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
             s_acc[1] = zero16;
         }
         if (HAS_P2C) {
-            const uint32_t paddr = lds_addr(&sm.p[32 * w + il + 63 + 4 * hh * (PS - 1)]);
+            // Element (key j, query il) is P'[j][X - j], X = 32w + il + 63: from one key to the next the bf16 index moves
+            // by PS - 1 (odd), so the element alternates between the low and the high half of its dword with the
+            // parity of j, starting from the parity of il.  The dwords of keys j and j + 2 are (PS - 1) dwords apart
+            // and are read with one two-address read; the unwanted half (a neighbouring, finite P' value) is
+            // multiplied by zero in the dot product that adds the wanted half to the score.
+            constexpr int PD = PS - 1;            // dwords between the elements of keys j and j + 2
+            const int X = 32 * w + il + 63, pl = X & 1;
+            const uint32_t pbase = lds_addr(sm.p) + 2 * (X - pl) + 2 * 4 * hh * PD;   // even keys: dword of element (4hh, X - 4hh)
+            const uint32_t pbase_odd = pbase + 2 * PD - 2 + 4 * pl;                 // odd keys
+            const bf16x2 sel_lo = {(__bf16)1.0f, (__bf16)0.0f}, sel_hi = {(__bf16)0.0f, (__bf16)1.0f};
+            const bf16x2 sel_even = pl ? sel_hi : sel_lo, sel_odd = pl ? sel_lo : sel_hi;
             uint32_t g[2][16];
-            static_for<32>([&](auto ec) {
-                constexpr int jt = decltype(ec)::value >> 4, e = decltype(ec)::value & 15;
-                constexpr int jc = 32 * jt + 8 * (e >> 2) + (e & 3);
-                g[jt][e] = lds_read_u16<2 * jc * (PS - 1)>(paddr);
+            static_for<16>([&](auto pc) {
+                constexpr int pr = decltype(pc)::value, jt = pr >> 3, grp = (pr >> 1) & 3, odd = pr & 1;
+                constexpr int e = 4 * grp + odd;              // elements e and e + 2: keys jc and jc + 2
+                constexpr int jc = 32 * jt + 8 * grp + odd;
+                const uint32_t addr = (odd ? pbase_odd : pbase) + 2 * (jc - odd) * PD;
+                const u32x2 t = lds_read2_u32<0, PD>(addr);
+                g[jt][e] = t[0];
+                g[jt][e + 2] = t[1];
             });
             lds_wait(g[0]);
             lds_wait(g[1]);
@@ -726,8 +746,9 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
 #pragma unroll
             for (int jt = 0; jt < 2; ++jt)
 #pragma unroll
-                for (int e = 0; e < 16; ++e)   // bf16 pair (value, 0) . (1, 1) + acc
-                    s_acc[jt][e] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, g[jt][e]), ones, s_acc[jt][e], false);
+                for (int e = 0; e < 16; ++e)
+                    s_acc[jt][e] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, g[jt][e]), (e & 1) ? sel_odd : sel_even,
+                                                                   s_acc[jt][e], false);
         }
         TDB_STAMP(1);
         phase_barrier();                  // scratch is free again; keys of step s+1 and values of step s are staged
