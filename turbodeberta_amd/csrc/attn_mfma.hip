@@ -193,22 +193,23 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         tile_id = v - hd * tiles_x;
         return true;
     };
-    // Packed launches: every wave keeps the boundaries of the first 64 sequences (one per lane), so that looking a
-    // tile up reads nothing from memory for batches of up to 64 sequences.
-    int cu_lo = 0, cu_hi = 0;
+    // Every wave keeps the lengths (fixed layout) or boundaries (packed) of the first 64 sequences, one per lane, so
+    // that looking a tile up reads nothing from memory for batches of up to 64 sequences: a lookup that waits for a
+    // load would also wait for every prefetch in flight (one in-order counter).
+    int cu_lo = 0, cu_hi = 0, len_lane = p.L;
     if (p.varlen) {
         cu_lo = p.cu_seqlens[min(l, p.B)];
         cu_hi = p.cu_seqlens[min(l + 1, p.B)];
+    } else if (p.seqlens) {
+        len_lane = p.seqlens[min(l, p.B - 1)];
     }
-    // tile_id -> (sequence, first row, valid length, first token): same map as tdb_locate_tile, with the packed
-    // boundaries of the first chunk out of registers and the sequence length of sequence pf_b given as pf_len
-    // (read ahead of time by the caller; pf_b = -1: none).
-    auto locate = [&](int tile_id, int pf_b, int pf_len, int& bb, int& r0, int& ln, int64_t& t0) {
+    // tile_id -> (sequence, first row, valid length, first token): same map as tdb_locate_tile
+    auto locate = [&](int tile_id, int& bb, int& r0, int& ln, int64_t& t0) {
         if (!p.varlen) {
             const int tiles = (p.L + BM - 1) / BM;
             bb = tile_id / tiles;
             r0 = (tile_id - bb * tiles) * BM;
-            const int raw = p.seqlens ? (bb == pf_b ? __builtin_amdgcn_readfirstlane(pf_len) : p.seqlens[bb]) : p.L;
+            const int raw = !p.seqlens ? p.L : bb < 64 ? __builtin_amdgcn_readlane(len_lane, bb) : p.seqlens[bb];
             ln = min(max(raw, 0), p.L);
             t0 = 0;
             return true;
@@ -249,7 +250,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     // First tile with live query rows among the virtual blocks vb, vb + gridDim.x, ...; vb = -1 if there is none.
     // Tiles that hold only padded query rows (fixed layout) get their zeros here, from whoever looks them up:
     // every wave of the workgroup walks the same list, each thread fills its share.
-    auto find_tile = [&](int vb, int pf_b, int pf_len) {
+    auto find_tile = [&](int vb) {
         Tile t;
         t.vb = -1;
         t.head = t.b = t.row0 = t.len = 0;
@@ -259,7 +260,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
             if (!tile_index(vb, hd, tile_id)) continue;
             int bb, r0, ln;
             int64_t t0;
-            if (!locate(tile_id, pf_b, pf_len, bb, r0, ln, t0)) continue;
+            if (!locate(tile_id, bb, r0, ln, t0)) continue;
             if (r0 >= ln) {
                 uint16_t* Oz = static_cast<uint16_t*>(p.o) + (p.varlen ? t0 * p.os_l : int64_t(bb) * p.os_b) + int64_t(hd) * p.os_h;
                 const int rows = min(BM, (p.varlen ? ln : p.L) - r0);
@@ -277,27 +278,13 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         }
         return t;
     };
-    // Sequence length of the tile of virtual block vb, requested ahead of its lookup (fixed layout).  It is read
-    // through the vector memory path on purpose: a scalar read would be waited for at the next workgroup barrier
-    // (LDS and scalar memory share a counter), a vector read is only waited for where its value is used.
-    auto length_ahead = [&](int vb, int& pf_b, int& pf_len) {
-        pf_b = -1;
-        pf_len = 0;
-        int hd, tile_id;
-        if (!p.varlen && p.seqlens && tile_index(vb, hd, tile_id)) {
-            pf_b = tile_id / ((p.L + BM - 1) / BM);
-            int idx = pf_b;
-            asm volatile("" : "+v"(idx));
-            pf_len = p.seqlens[idx];
-        }
-    };
     auto k_of = [&](const Tile& t) {
         return static_cast<const uint16_t*>(p.k) + (p.varlen ? t.tok0 * p.ks_l : int64_t(t.b) * p.ks_b) + int64_t(t.head) * p.ks_h;
     };
     auto pk_of = [&](const Tile& t) { return HAS_C2P ? static_cast<const uint16_t*>(p.pk) + int64_t(t.head) * p.pks_h : nullptr; };
     auto pq_of = [&](const Tile& t) { return HAS_P2C ? static_cast<const uint16_t*>(p.pq) + int64_t(t.head) * p.pqs_h : nullptr; };
 
-    Tile cur = find_tile(blockIdx.x, -1, 0);
+    Tile cur = find_tile(blockIdx.x);
     if (cur.vb < 0) return;
 
     // ---- pipeline of one tile -----------------------------------------------------------------------------------
@@ -467,18 +454,10 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
                 for (int rt = 0; rt < 3; ++rt) res[rt] = chain(fr[rt], qb);
             }
             if (HAS_P2C) {
-                bf16x8 kx[4];
-#pragma unroll
-                for (int c = 0; c < 4; ++c) {   // key tile (w & 1), chosen without indexing registers
-                    const u32x4 x0 = __builtin_bit_cast(u32x4, kb[0][c]), x1 = __builtin_bit_cast(u32x4, kb[1][c]);
-                    u32x4 r;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) r[e] = (w & 1) ? x1[e] : x0[e];
-                    kx[c] = __builtin_bit_cast(bf16x8, r);
-                }
                 res[3] = chain(fq[0], kb[0]);
                 res[4] = chain(fq[0], kb[1]);
-                res[5] = chain(fq[1], kx);
+                if (w & 1) res[5] = chain(fq[1], kb[1]);   // key tile (w & 1): a wave-uniform branch, no register copies
+                else res[5] = chain(fq[1], kb[0]);
             }
         };
         auto put_results = [&]() {
@@ -562,15 +541,10 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
             dl_step[s1][1] = dl_cold[s1][1];
         }
         TDB_T_DECL
+        phase_barrier();                  // first stage of the first tile is in LDS
         while (true) {
             TDB_PRESET;
             bind_tables();
-            // The tile after this one is looked up here, where the wait for its sequence length falls into the
-            // wait for the score waves; its delta values are read in the last step but one (when the fragment and
-            // result registers are no longer needed), its first stage during the last step.
-            int pf_b, pf_len;             // asked for here, used by the lookup after the opening barriers
-            length_ahead(cur.vb + gridDim.x, pf_b, pf_len);
-            phase_barrier();              // first stage of the tile is in LDS
             TDB_PSTAMP(1);
             // products of step 0; window rows of step 1 (they overwrite rows step 0 is done with); fragments of
             // step 1; prefetch for half A of step 0
@@ -595,9 +569,12 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
             TDB_PSTAMP(5);
             load_frags(off1, 1);
             TDB_PSTAMP(6);
-            // The tile after this one: its delta values are read in the last step but one (when the fragment and
-            // result registers are no longer needed), its first stage during the last step.
-            const Tile nxt = find_tile(cur.vb + gridDim.x, pf_b, pf_len);
+            // The tile after this one.  Its delta values are read at the end of the last step but one (when the fragment
+            // and result registers are no longer needed); its first LDS stage is read from global memory and written
+            // to LDS in half A of the last step, where this role has nothing else to do: after the barrier that ends
+            // that half, it is already at the next tile's first position products while the score waves finish the
+            // last step.
+            const Tile nxt = find_tile(cur.vb + gridDim.x);
             TDB_PSTAMP(7);
 
             int off2 = prev_off(off1);    // ring offset of step s+2
@@ -607,8 +584,8 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
                 TDB_STAMP(0);
                 products();               // of step s+1, into registers; issued first: the wait for the
                 __builtin_amdgcn_sched_barrier(0);  // prefetched global data then passes under the MFMAs
-                store(off2);              // new window rows of step s+2
                 if (!TAIL) {
+                    store(off2);          // new window rows of step s+2
                     fetch();              // window rows of step s+3: a full step ahead of their store
                     fetch_delta(s + 4);
                 }
@@ -616,26 +593,32 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
                 phase_barrier();          // score waves are done with the scratch; the staged tiles are visible
                 TDB_STAMP(2);
                 put_results();            // of step s+1
-                if (!TAIL) load_frags(off2, s & 1);  // of step s+2
+                if (!TAIL) {
+                    load_frags(off2, s & 1);  // of step s+2
+                } else {
+                    read_deltas(nxt);
+                }
                 off2 = prev_off(off2);
                 TDB_STAMP(3);
             };
             if (nsteps >= 2) {
                 for (int s = 0; s + 2 < nsteps; ++s) pos_step(s, std::false_type{});
                 pos_step(nsteps - 2, std::true_type{});
+            } else {
+                read_deltas(nxt);
             }
-            read_deltas(nxt);
-            // last key step: nothing left to prepare for this tile; the first stage of the next tile is requested
+            // Last key step: nothing left to prepare for this tile.  The ring, both key buffers and the Q fragment
+            // registers are free, so the next tile moves in; the barrier that ends this half is also the barrier
+            // after which the next tile's first stage is in LDS.
             phase_barrier();
             TDB_STAMP(0);
             read_stage(nxt);
             load_q(qb_next, nxt);
+            if (nxt.vb >= 0) write_stage();
             TDB_STAMP(1);
             phase_barrier();
             TDB_STAMP(2);
             if (nxt.vb < 0) break;
-            write_stage();                // (the score waves are still in half B of the last step: they read only V)
-            TDB_PSTAMP(0);
             cur = nxt;
             bind(cur);
 #pragma unroll
@@ -684,10 +667,10 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
             pre_v[n] = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, vvoff[n], 0, 0);
         }
     };
-    auto store_kv = [&](int kbuf) {
+    auto store_kv = [&](int kbuf, bool with_keys) {
 #pragma unroll
         for (int n = 0; n < 2; ++n) {
-            *reinterpret_cast<u32x4*>(&sm.k[kbuf][(srow + 32 * n) * RS + sch * 8]) = pre_k[n];
+            if (with_keys) *reinterpret_cast<u32x4*>(&sm.k[kbuf][(srow + 32 * n) * RS + sch * 8]) = pre_k[n];
             *reinterpret_cast<u32x4*>(&sm.v[(srow + 32 * n) * RS + sch * 8]) = pre_v[n];
         }
     };
@@ -701,7 +684,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         // ---- half A: keys of step s+2 and values of step s go to LDS (prefetched registers, nothing waits);
         //      position terms of step s out of the scratch.  Element (jj, i) of the score tile takes
         //      C'[i][i-jj+63] (fp32, straight into the accumulator) and P'[jj][32w+i-jj+63] (bf16) ----------------
-        store_kv(s & 1);
+        store_kv(s & 1, s + 2 < nsteps);  // (in the last step the key buffers already take the next tile's keys)
         f32x16 s_acc[2];
         if (HAS_C2P) {
             // float index of element e of key tile jt:  il*CS + il + 63 - 4*hh - jc,  jc = 32*jt + 8*(e>>2) + (e&3) <= 59
@@ -760,7 +743,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
 #pragma unroll
             for (int jt = 0; jt < 2; ++jt) s_acc[jt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[jt][c], qb[c], s_acc[jt], 0, 0, 0);
         load_kf((s + 1) & 1);             // K fragments of step s+1 (the MFMAs above have read this step's)
-        fetch_kv(s + 3, s + 1);           // for the next half A
+        if (s + 1 < nsteps) fetch_kv(s + 3, s + 1);   // for the next half A (nothing left to fetch in the last step)
         // V^T fragments through the transposing LDS read: the lane provides the address of 4 dims of one key
         bf16x8 vf[2][2][2];               // [key tile][16-key chunk][dim tile]
         {
@@ -834,12 +817,10 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     };
 
     // Opening of a tile, after its first barrier (first stage in LDS).  Everything that reads global memory is
-    // requested here and waited for much later: keys of step 2 / values of step 0 (stored in half A of step 0), the
-    // sequence length and Q fragments of the tile after this one.  The output rows of the previous tile are written
+    // requested here and waited for much later: keys of step 2 / values of step 0 (stored in half A of step 0) and
+    // the Q fragments of the tile after this one.  The output rows of the previous tile are written
     // last: stores count on the same in-order counter as loads, so a wait for any load issued after them would
     // also wait for them.
-    int pf_b, pf_len;                     // sequence length of the next tile, asked for one tile ahead of its lookup
-    length_ahead(cur.vb + gridDim.x, pf_b, pf_len);
     Tile nxt;
     bf16x8 qb_next[4];
     u32x2 o_out[2][4];                    // packed output rows of the tile just finished
@@ -848,13 +829,8 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     auto open_tile = [&]() {
         TDB_PRESET;
         load_kf(0);
-        TDB_PSTAMP(0);
-        nxt = find_tile(cur.vb + gridDim.x, pf_b, pf_len);
-        TDB_PSTAMP(1);
-        length_ahead(nxt.vb >= 0 ? nxt.vb + gridDim.x : nblocks, pf_b, pf_len);
         fetch_kv(2, 0);
-        load_q(qb_next, nxt);
-        TDB_PSTAMP(2);
+        TDB_PSTAMP(0);
         if (o_write) {
 #pragma unroll
             for (int dt = 0; dt < 2; ++dt)
@@ -866,6 +842,11 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         TDB_PSTAMP(4);
         phase_barrier();
         TDB_PSTAMP(5);
+        // the tile after this one is looked up while the position waves get step 1 ready
+        nxt = find_tile(cur.vb + gridDim.x);
+        TDB_PSTAMP(1);
+        load_q(qb_next, nxt);
+        TDB_PSTAMP(2);
     };
     // epilogue of a tile: normalised output rows, packed; lane holds d = 32*dt + 8*a + 4*hh + 0..3 of query row il
     auto close_tile = [&]() {
@@ -895,11 +876,9 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         for (int s = 0; s < nfull; ++s) key_step(s, std::false_type{});
         if (nfull < nsteps) key_step(nfull, std::true_type{});
 
-        // The position waves have put the first stage of the next tile into LDS in the meantime and go on to its
-        // first position products; this tile is closed under those.
+        // The position waves put the first stage of the next tile into LDS during the last step and are at its
+        // first position products by now; this tile is closed under those.
         TDB_PRESET;
-        if (nxt.vb >= 0) phase_barrier();
-        TDB_PSTAMP(6);
         close_tile();
         TDB_PSTAMP(7);
         TDB_STAMP(5);
