@@ -134,3 +134,38 @@ def test_config5_long_context_l4096():
     ref1 = O.attention(f(q), f(k), f(v), pk.float().cpu(), pq.float().cpu(), None,
                        position_buckets=BUCKETS, max_relative_positions=MAX_REL)[0]
     assert_close_bf16(outv[s:e].permute(1, 0, 2), ref1, "config 5 packed", tol=1e-2)
+
+
+def test_persistent_tile_walk_mixed_lengths():
+    """More tiles than workgroups, with everything a persistent workgroup can meet on its list: single-step tiles
+    (length <= 64), tiles with only padded rows (in the middle and at the end of a list), a sequence of length 0,
+    lengths on and next to tile and key-step boundaries, more than 64 sequences (lengths beyond the ones kept in
+    lane registers).  Checked against the vector-ALU kernel on the whole tensor, the oracle on a sample, and the
+    packed run (one workgroup per tile) bit for bit."""
+    B, L, heads = 72, 512, 4
+    base = [1, 2, 17, 63, 64, 65, 127, 128, 129, 191, 192, 193, 255, 256, 257, 300, 383, 384, 385, 448, 511, 512, 0, 5]
+    lengths = np.array((base * 3)[:B])
+    np.random.RandomState(3).shuffle(lengths)
+    q, k, v, pk, pq = _projected(B, L, heads=heads, seed=5)
+    lens = torch.from_numpy(lengths.astype(np.int32)).to(DEV)
+    print("[case] persistent walk, matrix-core kernel", flush=True)
+    out = flash_attention_with_disentangled(q, k, v, None, None, False, SCALE, BUCKETS, MAX_REL,
+                                            pos_key_layer=pk, pos_query_layer=pq, seqlens_k=lens)
+    torch.cuda.synchronize()
+    pad = torch.arange(L, device=DEV)[None, :] >= lens[:, None]
+    assert torch.all(out.permute(0, 2, 1, 3)[pad] == 0)
+    assert torch.isfinite(out.float()).all()
+    print("[case] persistent walk, vector-ALU kernel", flush=True)
+    gen = flash_attention_with_disentangled(q, k, v, None, None, False, SCALE, BUCKETS, MAX_REL, pos_key_layer=pk,
+                                            pos_query_layer=pq, seqlens_k=lens, force_generic=True)
+    assert (out.float() - gen.float()).abs().max().item() <= 1e-2
+    for n in (1, 64, 65, 129, 512):
+        b = int(np.flatnonzero(lengths == n)[-1])
+        assert_close_bf16(out[b, :, :n], _oracle_rows(q, k, v, pk, pq, b, n), f"walk seq {b} len {n}", tol=1e-2)
+    valid = ~pad
+    pack = lambda t: t.permute(0, 2, 1, 3)[valid].contiguous()
+    cu = torch.from_numpy(np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)).to(DEV)
+    print("[case] persistent walk, packed", flush=True)
+    outv = flash_attention_with_disentangled_varlen(pack(q), pack(k), pack(v), None, None, cu, cu, L, L, False, SCALE,
+                                                    BUCKETS, MAX_REL, pos_key_layer=pk, pos_query_layer=pq)
+    assert torch.equal(outv, pack(out))
