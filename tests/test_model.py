@@ -140,3 +140,43 @@ def test_bf16_encoder_matches_hf_eager_on_device():
     assert err_ours.mean().item() <= 1.25 * err_hf.mean().item() + 1e-4, (err_ours.mean().item(), err_hf.mean().item())
     assert err_ours.max().item() <= 1.5 * err_hf.max().item() + 1e-3, (err_ours.max().item(), err_hf.max().item())
     assert (a[valid] - b[valid]).abs().max().item() <= 1e-1
+
+
+@pytest.mark.gpu
+def test_eval_caches_follow_weight_updates():
+    """Eval-mode caches (position tables, fused Q/K/V weight, lengths): the cached forward equals the uncached one
+    (grad mode on takes the per-call path), a repeated call hits the caches and gives the same bits, and an in-place
+    weight update or a new mask invalidates them."""
+    cfg = _tiny()
+    model = FlashDebertaV2Model(cfg).eval()
+    fill_params(model)
+    model = model.to("cuda:0")
+    ids, mask = tiny_model_inputs()
+    ids, mask = torch.from_numpy(ids).cuda(), torch.from_numpy(mask).cuda()
+    att = model.encoder.layer[0].attention.self
+    print("[case] eval caches", flush=True)
+    uncached = model(input_ids=ids, attention_mask=mask).last_hidden_state.detach()     # grad mode on: no caches
+    assert "_tdb_tables" not in att.__dict__ and "_tdb_qkv" not in att.__dict__
+    with torch.no_grad():
+        first = model(input_ids=ids, attention_mask=mask).last_hidden_state
+        assert "_tdb_tables" in att.__dict__ and "_tdb_qkv" in att.__dict__
+        tables = att.__dict__["_tdb_tables"][1][0]
+        second = model(input_ids=ids, attention_mask=mask).last_hidden_state
+        assert att.__dict__["_tdb_tables"][1][0] is tables                               # cache hit
+    valid = mask.bool()
+    assert torch.equal(first, second)
+    assert (first[valid] - uncached[valid]).abs().max() <= 1e-5 * uncached[valid].abs().max()
+    with torch.no_grad():
+        att.key_proj.weight.mul_(1.5)                                                    # bumps the version counter
+        changed = model(input_ids=ids, attention_mask=mask).last_hidden_state
+        assert att.__dict__["_tdb_tables"][1][0] is not tables
+    fresh = model(input_ids=ids, attention_mask=mask).last_hidden_state.detach()
+    assert (changed[valid] - fresh[valid]).abs().max() <= 1e-5 * fresh[valid].abs().max()
+    assert (changed[valid] - first[valid]).abs().max() > 1e-3
+    with torch.no_grad():                                                                # shorter sequences, new mask
+        mask2 = mask.clone()
+        mask2[:, -3:] = 0
+        a = model(input_ids=ids, attention_mask=mask2).last_hidden_state
+    b = model(input_ids=ids, attention_mask=mask2).last_hidden_state.detach()
+    v2 = mask2.bool()
+    assert (a[v2] - b[v2]).abs().max() <= 1e-5 * b[v2].abs().max()

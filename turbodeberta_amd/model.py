@@ -13,7 +13,13 @@ What differs from the reference glue (model.py:34-186):
   ``[B, L, H*D]`` is a view;
 * padding is handled by per-sequence lengths inside the fixed-length kernel: no un-pad / re-pad
   gathers (model.py:138-183) and no host synchronisation (model.py:55-63, padding.py:82);
-* the position index is Hugging Face's for both terms (modeling_deberta_v2.py:318, :336-343).
+* the position index is Hugging Face's for both terms (modeling_deberta_v2.py:318, :336-343);
+* in eval mode, work that does not depend on the input is done once instead of once per call: the
+  per-head position tables (a function of the layer's weights and the shared relative embeddings
+  only; the reference recomputes both strip GEMMs every call, model.py:94-110) and the
+  concatenated Q/K/V weight of the single fused projection GEMM; the valid lengths are computed by
+  the first layer that sees a mask and reused by the others (the reference recomputes them, with
+  a host synchronisation, in every layer: model.py:55-63).
 """
 from __future__ import annotations
 
@@ -32,6 +38,26 @@ from transformers.models.deberta_v2.modeling_deberta_v2 import (
 
 from .ops.flash_attention import flash_attention_with_disentangled
 from .padding import key_padding_mask
+
+
+def _versions(*tensors):
+    """Identity of a set of tensors for cache keys: storage address and in-place modification counter."""
+    return tuple((t.data_ptr(), t._version, t.dtype, t.device) if t is not None else None for t in tensors)
+
+
+def _lengths_of(attention_mask):
+    """int32 [B] valid lengths of a right-padded batch.  The result is attached to the mask tensor, so the
+    layers of an encoder, which all receive the same mask object (modeling_deberta_v2.py:651-660), compute it
+    once per forward."""
+    cached = getattr(attention_mask, "_tdb_lengths", None)
+    if cached is not None and cached[0] == attention_mask._version:
+        return cached[1]
+    lengths = key_padding_mask(attention_mask).sum(dim=-1, dtype=torch.int32)
+    try:
+        attention_mask._tdb_lengths = (attention_mask._version, lengths)
+    except AttributeError:      # tensor subclasses without a __dict__
+        pass
+    return lengths
 
 
 class FlashDisentangledSelfAttention(DisentangledSelfAttention):
@@ -57,10 +83,17 @@ class FlashDisentangledSelfAttention(DisentangledSelfAttention):
         if query_states.shape[1] != L:
             raise ValueError("self-attention only: query_states and hidden_states must have one length")
 
-        heads = lambda x: x.view(B, L, H, D).permute(0, 2, 1, 3)          # [B, H, L, D] view, token-major storage
-        q = heads(self.query_proj(query_states))
-        k = heads(self.key_proj(hidden_states))
-        v = heads(self.value_proj(hidden_states))
+        frozen = not self.training and not torch.is_grad_enabled()       # nothing below can change between calls
+        if frozen and query_states is hidden_states:
+            # one projection GEMM; q, k, v are views into its [B, L, 3, H, D] output (token stride 3*H*D)
+            w, b = self._fused_qkv()
+            qkv = nn.functional.linear(hidden_states, w, b).view(B, L, 3, H, D)
+            q, k, v = (qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+        else:
+            heads = lambda x: x.view(B, L, H, D).permute(0, 2, 1, 3)      # [B, H, L, D] view, token-major storage
+            q = heads(self.query_proj(query_states))
+            k = heads(self.key_proj(hidden_states))
+            v = heads(self.value_proj(hidden_states))
 
         scale_factor = 1 + int("c2p" in self.pos_att_type) + int("p2c" in self.pos_att_type)
         pos_key = pos_query = None
@@ -68,24 +101,58 @@ class FlashDisentangledSelfAttention(DisentangledSelfAttention):
         if self.relative_attention:
             buckets, max_rel = self.position_buckets, self.max_relative_positions
             span = self.pos_ebd_size
-            rel = self.pos_dropout(rel_embeddings)[0:2 * span]                                   # HF:295
-            table = lambda proj: proj(rel).view(2 * span, H, D).permute(1, 0, 2)                 # [H, 2*span, D] view
-            if "c2p" in self.pos_att_type:
-                pos_key = table(self.key_proj if self.share_att_key else self.pos_key_proj)      # HF:296-312
-            if "p2c" in self.pos_att_type:
-                pos_query = table(self.query_proj if self.share_att_key else self.pos_query_proj)
+            if frozen:
+                pos_key, pos_query = self._position_tables(rel_embeddings, hidden_states.dtype)
+            else:
+                pos_key, pos_query = self._project_tables(self.pos_dropout(rel_embeddings)[0:2 * span])   # HF:295
         else:
             scale_factor = 1
         sm_scale = 1.0 / math.sqrt(D * scale_factor)                                             # HF:120-121, :243
 
-        seqlens = None
-        if attention_mask is not None:
-            seqlens = key_padding_mask(attention_mask).sum(dim=-1, dtype=torch.int32)
+        seqlens = _lengths_of(attention_mask) if attention_mask is not None else None
         out = flash_attention_with_disentangled(q, k, v, None, None, False, sm_scale, buckets, max_rel,
                                                 pos_key_layer=pos_key, pos_query_layer=pos_query,
                                                 seqlens_k=seqlens)
-        # out has q's strides: [B, H, L, D] view of token-major [B, L, H, D] storage
+        # out has q's strides: [B, H, L, D] view of token-major storage
         return (out.permute(0, 2, 1, 3).reshape(B, L, H * D), None)
+
+    def _project_tables(self, rel):
+        """Per-head projections of the relative embeddings, ``[H, 2*span, D]`` views (modeling_deberta_v2.py:296-312)."""
+        H, D = self.num_attention_heads, self.attention_head_size
+        table = lambda proj: proj(rel).view(rel.shape[0], H, D).permute(1, 0, 2)
+        pos_key = pos_query = None
+        if "c2p" in self.pos_att_type:
+            pos_key = table(self.key_proj if self.share_att_key else self.pos_key_proj)
+        if "p2c" in self.pos_att_type:
+            pos_query = table(self.query_proj if self.share_att_key else self.pos_query_proj)
+        return pos_key, pos_query
+
+    def _position_tables(self, rel_embeddings, dtype):
+        """Eval-mode cache of ``_project_tables``: recomputed only when the relative embeddings or the
+        projection weights have been modified (or moved / cast)."""
+        kp = self.key_proj if self.share_att_key else getattr(self, "pos_key_proj", None)
+        qp = self.query_proj if self.share_att_key else getattr(self, "pos_query_proj", None)
+        key = (_versions(rel_embeddings, *(t for m in (kp, qp) if m is not None for t in (m.weight, m.bias))), dtype)
+        cached = self.__dict__.get("_tdb_tables")
+        if cached is None or cached[0] != key:
+            rel = rel_embeddings[0:2 * self.pos_ebd_size]                # dropout is the identity in eval mode
+            cached = (key, self._project_tables(rel))
+            self.__dict__["_tdb_tables"] = cached
+        return cached[1]
+
+    def _fused_qkv(self):
+        """Eval-mode cache of the concatenated ``[3*H*D, hidden]`` projection weight (and bias)."""
+        mods = (self.query_proj, self.key_proj, self.value_proj)
+        key = _versions(*(t for m in mods for t in (m.weight, m.bias)))
+        cached = self.__dict__.get("_tdb_qkv")
+        if cached is None or cached[0] != key:
+            w = torch.cat([m.weight for m in mods], dim=0)
+            b = torch.cat([m.bias for m in mods], dim=0) if all(m.bias is not None for m in mods) else None
+            if b is None and any(m.bias is not None for m in mods):
+                b = torch.cat([m.bias if m.bias is not None else m.weight.new_zeros(m.weight.shape[0]) for m in mods])
+            cached = (key, (w, b))
+            self.__dict__["_tdb_qkv"] = cached
+        return cached[1]
 
 
 class FlashDebertaV2Attention(DebertaV2Attention):
