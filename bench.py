@@ -144,6 +144,49 @@ def cpu_baseline(tensors, lengths, budget_s=12.0):
                       f"float32 torch-CPU oracle, median of {len(times)} runs"}
 
 
+def model_benchmark(dev, steps=10, warmup=3):
+    """End-to-end forward of a DeBERTa-v3-large-shaped model (24 layers x 1024, 16 heads x 64, FFN 4096, vocabulary
+    128100, buckets 256, max_rel 512, shared keys, c2p|p2c, layer-normed relative embeddings; random N(0, 0.02)
+    weights, eval mode, bf16) on ids [16, 512] with right-padded lengths U[64, 512]: valid tokens per second with the
+    attention core on the fused kernel, and with Hugging Face's eager attention in the same model on the same GPU."""
+    from transformers import DebertaV2Config, DebertaV2Model
+    from turbodeberta_amd.model import patch_model
+    cfg = DebertaV2Config(vocab_size=128100, hidden_size=1024, num_hidden_layers=24, num_attention_heads=16,
+                          intermediate_size=4096, hidden_dropout_prob=0.0, attention_probs_dropout_prob=0.0,
+                          max_position_embeddings=512, type_vocab_size=0, relative_attention=True, position_buckets=256,
+                          max_relative_positions=512, share_att_key=True, pos_att_type=["c2p", "p2c"],
+                          norm_rel_ebd="layer_norm", position_biased_input=False, layer_norm_eps=1e-7,
+                          initializer_range=0.02)
+    torch.manual_seed(0)
+    with torch.device(dev):
+        model = DebertaV2Model(cfg)
+    model = model.to(torch.bfloat16).eval()
+    rs = np.random.RandomState(0)
+    lengths = rs.randint(64, 513, size=16)
+    ids = torch.from_numpy(rs.randint(0, 128000, size=(16, 512))).to(dev)
+    mask = torch.from_numpy((np.arange(512)[None] < lengths[:, None]).astype(np.int64)).to(dev)
+
+    def run(m):
+        with torch.no_grad():
+            for _ in range(warmup):
+                m(input_ids=ids, attention_mask=mask)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                m(input_ids=ids, attention_mask=mask)
+            torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / steps
+
+    t_eager = run(model)
+    t_fused = run(patch_model(model))
+    tokens = float(lengths.sum())
+    return {"workload": "v3-large-shaped model, ids [16, 512], lengths U[64,512] seed 0 (%d valid tokens), bf16" % int(tokens),
+            "steps": steps, "warmup": warmup,
+            "fused": {"ms_per_forward": round(t_fused * 1e3, 3), "valid_tokens_per_s": round(tokens / t_fused, 1)},
+            "hf_eager_same_gpu": {"ms_per_forward": round(t_eager * 1e3, 3), "valid_tokens_per_s": round(tokens / t_eager, 1)},
+            "speedup": round(t_eager / t_fused, 3)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -151,6 +194,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--workload", choices=["both", "fixed", "varlen"], default="both")
+    ap.add_argument("--with-model", action="store_true",
+                    help="add the end-to-end forward of a v3-large-shaped model (fused attention vs Hugging Face eager "
+                         "attention on the same GPU) to the JSON line as \"model\"")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one plain device copy of 512 MiB (read) + 512 MiB (write), the yardstick the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run are scaled by")
@@ -209,6 +255,10 @@ def main():
                          **res_var}
     if not args.no_cpu_baseline and tensors is not None:
         out["cpu_baseline"] = cpu_baseline(tensors, lengths_f)
+    if args.with_model:
+        del tensors
+        torch.cuda.empty_cache()
+        out["model"] = model_benchmark(dev)
     print(json.dumps(out))
 
 
