@@ -231,6 +231,27 @@ def test_bf16_varlen_vs_oracle(force_generic):
     assert_close_bf16(out.cpu(), ref, "bf16 varlen", tol=1e-2)
 
 
+@pytest.mark.parametrize("force_generic", [False, True])
+def test_bf16_varlen_more_than_64_sequences(force_generic):
+    """150 short sequences: the wave-wide scan over the packed boundaries needs three chunks of 64, of which only
+    the first is kept in registers by the matrix-core kernel."""
+    H, D, buckets, max_rel = 2, 64, 256, 512
+    rs = np.random.RandomState(4)
+    lengths = [int(x) for x in rs.randint(1, 200, size=150)]
+    lengths[70], lengths[140] = 0, 130
+    inp = make_inputs(11, len(lengths), H, max(lengths), D, buckets, max_rel, dtype=torch.bfloat16)
+    packed, cu = pack(inp, lengths)
+    f = lambda t: t.float()
+    ref = O.attention_varlen(f(packed["q"]), f(packed["k"]), f(packed["v"]), f(inp["pk"]), f(inp["pq"]), cu,
+                             position_buckets=buckets, max_relative_positions=max_rel)
+    print(f"[case] bf16 varlen 150 sequences generic={force_generic}", flush=True)
+    out = flash_attention_with_disentangled_varlen(
+        packed["q"].to(DEV), packed["k"].to(DEV), packed["v"].to(DEV), None, None, cu.to(DEV), cu.to(DEV),
+        max(lengths), max(lengths), False, 1 / math.sqrt(3 * D), buckets, max_rel,
+        pos_key_layer=inp["pk"].to(DEV), pos_query_layer=inp["pq"].to(DEV), force_generic=force_generic)
+    assert_close_bf16(out.cpu(), ref, "bf16 varlen, 150 sequences", tol=1e-2)
+
+
 def test_backward_raises_like_the_reference():
     q = torch.randn(1, 1, 8, 64, device=DEV, requires_grad=True)
     out = flash_attention_with_disentangled(q, q, q, None, None)

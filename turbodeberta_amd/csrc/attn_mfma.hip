@@ -71,47 +71,6 @@ __device__ __forceinline__ u32x2 pack4(float a, float b, float c, float d) {
     return r;
 }
 
-template <int... Is, typename F>
-__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, Is...>, F&& f) {
-    (f(std::integral_constant<int, Is>{}), ...);
-}
-// f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>): loop indices usable as immediates
-template <int N, typename F>
-__device__ __forceinline__ void static_for(F&& f) {
-    static_for_impl(std::make_integer_sequence<int, N>{}, static_cast<F&&>(f));
-}
-
-// Skewed LDS gathers, issued as inline asm with immediate offsets.  (Left to the compiler, runs of
-// neighbouring narrow reads get fused into 64-bit reads at 2- or 4-byte alignment, which this LDS
-// serialises lane by lane.)  Results are valid after lds_wait().
-template <int OFF0, int OFF1>   // two dwords at dword offsets OFF0, OFF1 from a 4-byte aligned address
-__device__ __forceinline__ float2 lds_read2_f32(uint32_t addr) {
-    float2 r;
-    asm volatile("ds_read2_b32 %0, %1 offset0:%2 offset1:%3" : "=v"(r) : "v"(addr), "n"(OFF0), "n"(OFF1) : "memory");
-    return r;
-}
-template <int OFF0, int OFF1>   // the same, as raw dwords
-__device__ __forceinline__ u32x2 lds_read2_u32(uint32_t addr) {
-    u32x2 r;
-    asm volatile("ds_read2_b32 %0, %1 offset0:%2 offset1:%3" : "=v"(r) : "v"(addr), "n"(OFF0), "n"(OFF1) : "memory");
-    return r;
-}
-template <int OFF>              // one zero-extended 16-bit value at byte offset OFF
-__device__ __forceinline__ uint32_t lds_read_u16(uint32_t addr) {
-    uint32_t r;
-    asm volatile("ds_read_u16 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF) : "memory");
-    return r;
-}
-__device__ __forceinline__ void lds_wait(f32x16& a, f32x16& b) {
-    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a), "+v"(b) : : "memory");
-}
-__device__ __forceinline__ void lds_wait(uint32_t (&g)[16]) {
-    asm volatile("s_waitcnt lgkmcnt(0)"
-                 : "+v"(g[0]), "+v"(g[1]), "+v"(g[2]), "+v"(g[3]), "+v"(g[4]), "+v"(g[5]), "+v"(g[6]), "+v"(g[7]),
-                   "+v"(g[8]), "+v"(g[9]), "+v"(g[10]), "+v"(g[11]), "+v"(g[12]), "+v"(g[13]), "+v"(g[14]), "+v"(g[15])
-                 :
-                 : "memory");
-}
 // Workgroup barrier that instruction scheduling may not move anything across either: register-only work (MFMAs,
 // address arithmetic) stays in the pipeline half it was written in.
 #ifdef TDB_TIMING
@@ -151,9 +110,6 @@ __device__ __forceinline__ void phase_barrier() {
     __builtin_amdgcn_sched_barrier(0);
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
-}
-__device__ __forceinline__ uint32_t lds_addr(const void* p) {
-    return uint32_t(uintptr_t(TDB_LDS(const char, p)));
 }
 
 template <bool HAS_C2P, bool HAS_P2C>
@@ -685,18 +641,17 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         //      position terms of step s out of the scratch.  Element (jj, i) of the score tile takes
         //      C'[i][i-jj+63] (fp32, straight into the accumulator) and P'[jj][32w+i-jj+63] (bf16) ----------------
         store_kv(s & 1, s + 2 < nsteps);  // (in the last step the key buffers already take the next tile's keys)
+        // The gathers are ordinary LDS loads of dwords at 4-byte alignment; the compiler pairs them into two-address
+        // reads and places the waits.  (Loads issued from inline assembly would be invisible to it: it may then copy
+        // a destination register before the data has arrived.)
         f32x16 s_acc[2];
         if (HAS_C2P) {
             // float index of element e of key tile jt:  il*CS + il + 63 - 4*hh - jc,  jc = 32*jt + 8*(e>>2) + (e&3) <= 59
-            const uint32_t caddr = lds_addr(&sm.c[w][il * (CS + 1) + 4 - 4 * hh]);
-            static_for<16>([&](auto pc) {
-                constexpr int pr = decltype(pc)::value, jt = pr >> 3, e = 2 * (pr & 7);
-                constexpr int jc = 32 * jt + 8 * (e >> 2) + (e & 3);
-                const float2 t = lds_read2_f32<59 - jc, 59 - jc - 1>(caddr);
-                s_acc[jt][e] = t.x;
-                s_acc[jt][e + 1] = t.y;
-            });
-            if (!HAS_P2C) lds_wait(s_acc[0], s_acc[1]);
+            const auto* cbase = TDB_LDS(const float, &sm.c[w][il * (CS + 1) + 4 - 4 * hh]);
+#pragma unroll
+            for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) s_acc[jt][e] = cbase[59 - (32 * jt + 8 * (e >> 2) + (e & 3))];
         } else {
             s_acc[0] = zero16;
             s_acc[1] = zero16;
@@ -705,27 +660,21 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
             // Element (key j, query il) is P'[j][X - j], X = 32w + il + 63: from one key to the next the bf16 index moves
             // by PS - 1 (odd), so the element alternates between the low and the high half of its dword with the
             // parity of j, starting from the parity of il.  The dwords of keys j and j + 2 are (PS - 1) dwords apart
-            // and are read with one two-address read; the unwanted half (a neighbouring, finite P' value) is
-            // multiplied by zero in the dot product that adds the wanted half to the score.
+            // (one two-address read); the unwanted half (a neighbouring, finite P' value) is multiplied by zero in
+            // the dot product that adds the wanted half to the score.
             constexpr int PD = PS - 1;            // dwords between the elements of keys j and j + 2
             const int X = 32 * w + il + 63, pl = X & 1;
-            const uint32_t pbase = lds_addr(sm.p) + 2 * (X - pl) + 2 * 4 * hh * PD;   // even keys: dword of element (4hh, X - 4hh)
-            const uint32_t pbase_odd = pbase + 2 * PD - 2 + 4 * pl;                 // odd keys
+            const auto* pbase = TDB_LDS(const uint32_t, sm.p) + (X - pl) / 2 + 2 * hh * PD;   // dword of element (4hh, X - 4hh)
             const bf16x2 sel_lo = {(__bf16)1.0f, (__bf16)0.0f}, sel_hi = {(__bf16)0.0f, (__bf16)1.0f};
             const bf16x2 sel_even = pl ? sel_hi : sel_lo, sel_odd = pl ? sel_lo : sel_hi;
             uint32_t g[2][16];
-            static_for<16>([&](auto pc) {
-                constexpr int pr = decltype(pc)::value, jt = pr >> 3, grp = (pr >> 1) & 3, odd = pr & 1;
-                constexpr int e = 4 * grp + odd;              // elements e and e + 2: keys jc and jc + 2
-                constexpr int jc = 32 * jt + 8 * grp + odd;
-                const uint32_t addr = (odd ? pbase_odd : pbase) + 2 * (jc - odd) * PD;
-                const u32x2 t = lds_read2_u32<0, PD>(addr);
-                g[jt][e] = t[0];
-                g[jt][e + 2] = t[1];
-            });
-            lds_wait(g[0]);
-            lds_wait(g[1]);
-            lds_wait(s_acc[0], s_acc[1]);
+#pragma unroll
+            for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const int jc = 32 * jt + 8 * (e >> 2) + (e & 3);
+                    g[jt][e] = (jc & 1) ? pbase[pl + (jc * PD - 1) / 2] : pbase[(jc / 2) * PD];
+                }
 #pragma unroll
             for (int jt = 0; jt < 2; ++jt)
 #pragma unroll
