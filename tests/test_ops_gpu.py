@@ -252,6 +252,42 @@ def test_bf16_varlen_more_than_64_sequences(force_generic):
     assert_close_bf16(out.cpu(), ref, "bf16 varlen, 150 sequences", tol=1e-2)
 
 
+@pytest.mark.parametrize("force_generic", [False, True])
+@pytest.mark.parametrize("B,H,L,buckets,max_rel,lengths", [
+    (2, 4, 512, 256, 512, (512, 389)),
+    (3, 1, 129, 256, 512, (129, 64, 3)),
+    (1, 2, 300, 32, 128, None),
+    (1, 1, 1100, 256, 512, None),
+])
+def test_fp16_fixed_vs_oracle(B, H, L, buckets, max_rel, lengths, force_generic):
+    """float16 inputs take the matrix-core kernel too (fp16 MFMA, fp32 accumulation); 11 significant bits give a
+    tighter bound than bfloat16."""
+    inp = make_inputs(12, B, H, L, 64, buckets, max_rel, dtype=torch.float16, lengths=lengths)
+    out = run_fixed(inp, buckets, max_rel, force_generic=force_generic)
+    assert out.dtype == torch.float16
+    ref32 = oracle_fixed(inp, buckets, max_rel, dtype=torch.float32)
+    assert_close_bf16(out, ref32, "fp16 vs fp32 oracle on rounded inputs", tol=2e-3)
+
+
+def test_fp16_varlen_matrix_core_equals_vector_alu():
+    H, D, buckets, max_rel = 4, 64, 256, 512
+    rs = np.random.RandomState(2)
+    lengths = [int(x) for x in rs.randint(16, 513, size=10)] + [1, 128, 129]
+    inp = make_inputs(13, len(lengths), H, max(lengths), D, buckets, max_rel, dtype=torch.float16)
+    packed, cu = pack(inp, lengths)
+    f = lambda t: t.float()
+    ref = O.attention_varlen(f(packed["q"]), f(packed["k"]), f(packed["v"]), f(inp["pk"]), f(inp["pq"]), cu,
+                             position_buckets=buckets, max_relative_positions=max_rel)
+    outs = []
+    for gen in (False, True):
+        print(f"[case] fp16 varlen generic={gen}", flush=True)
+        outs.append(flash_attention_with_disentangled_varlen(
+            packed["q"].to(DEV), packed["k"].to(DEV), packed["v"].to(DEV), None, None, cu.to(DEV), cu.to(DEV),
+            max(lengths), max(lengths), False, 1 / math.sqrt(3 * D), buckets, max_rel,
+            pos_key_layer=inp["pk"].to(DEV), pos_query_layer=inp["pq"].to(DEV), force_generic=gen).cpu())
+        assert_close_bf16(outs[-1], ref, f"fp16 varlen generic={gen}", tol=2e-3)
+
+
 def test_backward_raises_like_the_reference():
     q = torch.randn(1, 1, 8, 64, device=DEV, requires_grad=True)
     out = flash_attention_with_disentangled(q, q, q, None, None)

@@ -1,4 +1,4 @@
-// Matrix-core disentangled-attention forward for bf16, head_dim 64 (gfx950, wave64, MFMA 32x32x16).
+// Matrix-core disentangled-attention forward for bf16 and fp16, head_dim 64 (gfx950, wave64, MFMA 32x32x16).
 //
 // One workgroup = one tile of 128 query rows of one (sequence, head), walked over the keys 64 at a
 // time.  It has 8 waves in two roles, paired on the SIMDs so that their matrix and vector work
@@ -30,6 +30,8 @@ namespace {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(4))) short s16x4;
 typedef __attribute__((ext_vector_type(8))) short s16x8;
@@ -58,13 +60,37 @@ struct Smem {
     uint16_t p[BN * PS];
 };
 
-__device__ __forceinline__ bf16x8 lds_frag(const uint16_t* row_base, int row, int col) {
-    return *reinterpret_cast<const bf16x8*>(row_base + row * RS + col);
+// The two 16-bit element types the kernel is instantiated for: what differs is the MFMA, the dot-product
+// instruction and the float conversion.  (bf16: fp32's range, 8 significant bits; fp16: 11 bits, range 65504 --
+// the p2c products are stored in the element type, the probabilities are at most 2^8.)
+template <int DT>
+struct Elem;
+template <>
+struct Elem<TDB_BF16> {
+    using T = __bf16;
+    using X2 = bf16x2;
+    using X8 = bf16x8;
+    static __device__ __forceinline__ f32x16 mfma(X8 a, X8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+    static __device__ __forceinline__ float dot2(X2 a, X2 b, float c) { return __builtin_amdgcn_fdot2_f32_bf16(a, b, c, false); }
+};
+template <>
+struct Elem<TDB_F16> {
+    using T = _Float16;
+    using X2 = f16x2;
+    using X8 = f16x8;
+    static __device__ __forceinline__ f32x16 mfma(X8 a, X8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
+    static __device__ __forceinline__ float dot2(X2 a, X2 b, float c) { return __builtin_amdgcn_fdot2(a, b, c, false); }
+};
+
+template <typename X8>
+__device__ __forceinline__ X8 lds_frag(const uint16_t* row_base, int row, int col) {
+    return *reinterpret_cast<const X8*>(row_base + row * RS + col);
 }
 
+template <typename E>
 __device__ __forceinline__ u32x2 pack4(float a, float b, float c, float d) {
-    bf16x2 lo = {(__bf16)a, (__bf16)b};
-    bf16x2 hi = {(__bf16)c, (__bf16)d};
+    typename E::X2 lo = {(typename E::T)a, (typename E::T)b};
+    typename E::X2 hi = {(typename E::T)c, (typename E::T)d};
     u32x2 r;
     r[0] = __builtin_bit_cast(uint32_t, lo);
     r[1] = __builtin_bit_cast(uint32_t, hi);
@@ -112,8 +138,12 @@ __device__ __forceinline__ void phase_barrier() {
     __builtin_amdgcn_sched_barrier(0);
 }
 
-template <bool HAS_C2P, bool HAS_P2C>
+template <bool HAS_C2P, bool HAS_P2C, int DT>
 __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelParams p, const int nblocks) {
+    using E = Elem<DT>;
+    using ET = typename E::T;
+    using X2 = typename E::X2;
+    using X8 = typename E::X8;
     extern __shared__ __attribute__((aligned(16))) char smem_raw[];
     Smem& sm = *reinterpret_cast<Smem*>(smem_raw);
     constexpr bool HAS_POS = HAS_C2P || HAS_P2C;
@@ -282,15 +312,15 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     bind(cur);
 
     // Q^T fragments of query block w: B operand of S^T = K.Q^T (score wave) and of C'^T = K_r'.Q^T (position wave)
-    bf16x8 qb[4];
-    auto load_q = [&](bf16x8 (&dst)[4], const Tile& t) {
+    X8 qb[4];
+    auto load_q = [&](X8 (&dst)[4], const Tile& t) {
         const uint16_t* Qt = static_cast<const uint16_t*>(p.q) + (p.varlen ? t.tok0 * p.qs_l : int64_t(t.b) * p.qs_b) + int64_t(t.head) * p.qs_h;
         const int qrow = t.row0 + 32 * w + il;
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             u32x4 x = {0, 0, 0, 0};
             if (t.vb >= 0 && qrow < t.len) x = *reinterpret_cast<const u32x4*>(Qt + int64_t(qrow) * p.qs_l + 16 * c + 8 * hh);
-            dst[c] = __builtin_bit_cast(bf16x8, x);
+            dst[c] = __builtin_bit_cast(X8, x);
         }
     };
     load_q(qb, cur);
@@ -375,7 +405,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         //   products    c2p  C'^T[r, i] = K_r'[r].Q_i  (3 tiles),  p2c  P'^T[r, j] = Q_r'[r].K_j  (wave w: tile w
         //               against both key tiles, and tile (4 + w/2, w & 1)) -- 24 MFMAs;
         //   put_results c2p as fp32 C'[i][r'], p2c as bf16 P'[j][r''] into the scratch.
-        bf16x8 fr[3][4], fq[2][4], kb[2][4];
+        X8 fr[3][4], fq[2][4], kb[2][4];
         f32x16 res[6];
         auto load_frags = [&](int o, int kbuf) {
             auto ring = [&](int x) { const int t = x + o; return t >= WIN ? t - WIN : t; };
@@ -384,25 +414,25 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
                 for (int rt = 0; rt < 3; ++rt) {
                     const int row = ring(32 * w + 32 * rt + il);
 #pragma unroll
-                    for (int c = 0; c < 4; ++c) fr[rt][c] = lds_frag(sm.kr, row, 16 * c + 8 * hh);
+                    for (int c = 0; c < 4; ++c) fr[rt][c] = lds_frag<X8>(sm.kr, row, 16 * c + 8 * hh);
                 }
             }
             if (HAS_P2C) {
                 const int row3 = ring(32 * w + il), row4 = ring(32 * (4 + (w >> 1)) + il);
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
-                    fq[0][c] = lds_frag(sm.qr, row3, 16 * c + 8 * hh);
-                    fq[1][c] = lds_frag(sm.qr, row4, 16 * c + 8 * hh);
-                    kb[0][c] = lds_frag(sm.k[kbuf], il, 16 * c + 8 * hh);
-                    kb[1][c] = lds_frag(sm.k[kbuf], 32 + il, 16 * c + 8 * hh);
+                    fq[0][c] = lds_frag<X8>(sm.qr, row3, 16 * c + 8 * hh);
+                    fq[1][c] = lds_frag<X8>(sm.qr, row4, 16 * c + 8 * hh);
+                    kb[0][c] = lds_frag<X8>(sm.k[kbuf], il, 16 * c + 8 * hh);
+                    kb[1][c] = lds_frag<X8>(sm.k[kbuf], 32 + il, 16 * c + 8 * hh);
                 }
             }
         };
         auto products = [&]() {
-            auto chain = [&](const bf16x8 (&a)[4], const bf16x8 (&bb)[4]) {
-                f32x16 acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], bb[0], zero16, 0, 0, 0);
+            auto chain = [&](const X8 (&a)[4], const X8 (&bb)[4]) {
+                f32x16 acc = E::mfma(a[0], bb[0], zero16);
 #pragma unroll
-                for (int c = 1; c < 4; ++c) acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[c], bb[c], acc, 0, 0, 0);
+                for (int c = 1; c < 4; ++c) acc = E::mfma(a[c], bb[c], acc);
                 return acc;
             };
             if (HAS_C2P) {
@@ -430,7 +460,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
 #pragma unroll
                     for (int a = 0; a < 4; ++a)
                         *reinterpret_cast<u32x2*>(&sm.p[(32 * jt + il) * PS + 32 * rt + 8 * a + 4 * hh]) =
-                            pack4(acc[4 * a], acc[4 * a + 1], acc[4 * a + 2], acc[4 * a + 3]);
+                            pack4<E>(acc[4 * a], acc[4 * a + 1], acc[4 * a + 2], acc[4 * a + 3]);
                 };
                 put_p(w, 0, res[3]);
                 put_p(w, 1, res[4]);
@@ -443,7 +473,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         // the 64 new rows of steps 1 to 3), the row reads depend on them.
         int dl_win[WIN / 32], dl_step[3][2];
         u32x4 st_k[4], st_wk[WIN / 32], st_wq[WIN / 32];
-        bf16x8 qb_next[4];
+        X8 qb_next[4];
         // (Both readers assign every register also when there is no next tile: a conditional assignment would keep the
         // previous tile's values alive across the whole tile body.)
         auto read_deltas = [&](const Tile& t) {
@@ -587,16 +617,16 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
 
     // ===================================================== score waves ============================================
     const float c_exp = p.scale * 1.4426950408889634f;   // softmax in base 2
-    const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
+    const X2 ones = {(ET)1.0f, (ET)1.0f};
     f32x16 o_acc[2];
     float m_run, l_run;
 
-    bf16x8 kf[2][4];                      // K fragments: A operand of S^T = K.Q^T
+    X8 kf[2][4];                      // K fragments: A operand of S^T = K.Q^T
     auto load_kf = [&](int kbuf) {
 #pragma unroll
         for (int jt = 0; jt < 2; ++jt)
 #pragma unroll
-            for (int c = 0; c < 4; ++c) kf[jt][c] = lds_frag(sm.k[kbuf], 32 * jt + il, 16 * c + 8 * hh);
+            for (int c = 0; c < 4; ++c) kf[jt][c] = lds_frag<X8>(sm.k[kbuf], 32 * jt + il, 16 * c + 8 * hh);
     };
     // Keys and values travel global -> registers -> LDS through the score waves: thread tid stages chunk sch of rows
     // srow and srow + 32 of a 64-row step.  Buffer loads: the buffer of a step starts at its first row and ends with
@@ -665,8 +695,8 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
             constexpr int PD = PS - 1;            // dwords between the elements of keys j and j + 2
             const int X = 32 * w + il + 63, pl = X & 1;
             const auto* pbase = TDB_LDS(const uint32_t, sm.p) + (X - pl) / 2 + 2 * hh * PD;   // dword of element (4hh, X - 4hh)
-            const bf16x2 sel_lo = {(__bf16)1.0f, (__bf16)0.0f}, sel_hi = {(__bf16)0.0f, (__bf16)1.0f};
-            const bf16x2 sel_even = pl ? sel_hi : sel_lo, sel_odd = pl ? sel_lo : sel_hi;
+            const X2 sel_lo = {(ET)1.0f, (ET)0.0f}, sel_hi = {(ET)0.0f, (ET)1.0f};
+            const X2 sel_even = pl ? sel_hi : sel_lo, sel_odd = pl ? sel_lo : sel_hi;
             uint32_t g[2][16];
 #pragma unroll
             for (int jt = 0; jt < 2; ++jt)
@@ -679,8 +709,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
             for (int jt = 0; jt < 2; ++jt)
 #pragma unroll
                 for (int e = 0; e < 16; ++e)
-                    s_acc[jt][e] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, g[jt][e]), (e & 1) ? sel_odd : sel_even,
-                                                                   s_acc[jt][e], false);
+                    s_acc[jt][e] = E::dot2(__builtin_bit_cast(X2, g[jt][e]), (e & 1) ? sel_odd : sel_even, s_acc[jt][e]);
         }
         TDB_STAMP(1);
         phase_barrier();                  // scratch is free again; keys of step s+1 and values of step s are staged
@@ -690,11 +719,11 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
 #pragma unroll
         for (int c = 0; c < 4; ++c)
 #pragma unroll
-            for (int jt = 0; jt < 2; ++jt) s_acc[jt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[jt][c], qb[c], s_acc[jt], 0, 0, 0);
+            for (int jt = 0; jt < 2; ++jt) s_acc[jt] = E::mfma(kf[jt][c], qb[c], s_acc[jt]);
         load_kf((s + 1) & 1);             // K fragments of step s+1 (the MFMAs above have read this step's)
         if (s + 1 < nsteps) fetch_kv(s + 3, s + 1);   // for the next half A (nothing left to fetch in the last step)
         // V^T fragments through the transposing LDS read: the lane provides the address of 4 dims of one key
-        bf16x8 vf[2][2][2];               // [key tile][16-key chunk][dim tile]
+        X8 vf[2][2][2];               // [key tile][16-key chunk][dim tile]
         {
             const int g = l >> 4, ll = l & 15;
             const uint16_t* vbase = &sm.v[((ll >> 2) + 4 * (g >> 1)) * RS + 16 * (g & 1) + 4 * (ll & 3)];
@@ -708,7 +737,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
                         const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(TDB_LDS(s16x4, src));
                         const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(TDB_LDS(s16x4, src + 8 * RS));
                         const s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                        vf[jt][c][dt] = __builtin_bit_cast(bf16x8, both);
+                        vf[jt][c][dt] = __builtin_bit_cast(X8, both);
                     }
         }
         if (MASKED) {
@@ -751,15 +780,15 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
                 for (int h2 = 0; h2 < 4; ++h2) {
                     const float p0 = __builtin_amdgcn_exp2f(fmaf(s_acc[jt][8 * c + 2 * h2], c_exp, -mc));
                     const float p1 = __builtin_amdgcn_exp2f(fmaf(s_acc[jt][8 * c + 2 * h2 + 1], c_exp, -mc));
-                    const bf16x2 pr = {(__bf16)p0, (__bf16)p1};
-                    psum = __builtin_amdgcn_fdot2_f32_bf16(pr, ones, psum, false);   // sum of what the MFMA will see
+                    const X2 pr = {(ET)p0, (ET)p1};
+                    psum = E::dot2(pr, ones, psum);   // sum of what the MFMA will see
                     pw[h2] = __builtin_bit_cast(uint32_t, pr);
                 }
-                const bf16x8 pb = __builtin_bit_cast(bf16x8, u32x4{pw[0], pw[1], pw[2], pw[3]});
+                const X8 pb = __builtin_bit_cast(X8, u32x4{pw[0], pw[1], pw[2], pw[3]});
                 // O^T += V^T.P^T
 #pragma unroll
                 for (int dt = 0; dt < 2; ++dt)
-                    o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[jt][c][dt], pb, o_acc[dt], 0, 0, 0);
+                    o_acc[dt] = E::mfma(vf[jt][c][dt], pb, o_acc[dt]);
             }
         l_run += psum;
         TDB_STAMP(3);
@@ -771,7 +800,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     // last: stores count on the same in-order counter as loads, so a wait for any load issued after them would
     // also wait for them.
     Tile nxt;
-    bf16x8 qb_next[4];
+    X8 qb_next[4];
     u32x2 o_out[2][4];                    // packed output rows of the tile just finished
     uint16_t* o_ptr = nullptr;
     bool o_write = false;
@@ -810,7 +839,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
 #pragma unroll
             for (int a = 0; a < 4; ++a) {
                 u32x2 r = {0, 0};
-                if (live) r = pack4(o_acc[dt][4 * a] * inv, o_acc[dt][4 * a + 1] * inv, o_acc[dt][4 * a + 2] * inv, o_acc[dt][4 * a + 3] * inv);
+                if (live) r = pack4<E>(o_acc[dt][4 * a] * inv, o_acc[dt][4 * a + 1] * inv, o_acc[dt][4 * a + 2] * inv, o_acc[dt][4 * a + 3] * inv);
                 o_out[dt][a] = r;
             }
     };
@@ -852,9 +881,9 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
 }  // namespace
 
 bool tdb_mfma_supported(const TdbKernelParams& p, int dtype) {
-    // bf16, head_dim 64, position terms as fused tables (or none); strips go to the generic kernel.
+    // bf16 or fp16, head_dim 64, position terms as fused tables (or none); strips go to the generic kernel.
     // Buffer loads address rows with 32-bit byte offsets from the start of a (sequence, head).
-    if (dtype != TDB_BF16 || p.D != 64 || p.c2p || p.p2c) return false;
+    if ((dtype != TDB_BF16 && dtype != TDB_F16) || p.D != 64 || p.c2p || p.p2c) return false;
     const int64_t lim = int64_t(1) << 31;
     const int64_t rows = p.L;
     if (rows * p.ks_l * 2 >= lim || rows * p.vs_l * 2 >= lim) return false;
@@ -863,7 +892,7 @@ bool tdb_mfma_supported(const TdbKernelParams& p, int dtype) {
     return true;
 }
 
-hipError_t tdb_launch_mfma(const TdbKernelParams& p, int, hipStream_t stream) {
+hipError_t tdb_launch_mfma(const TdbKernelParams& p, int dtype, hipStream_t stream) {
     const int64_t tiles = int64_t(p.varlen ? p.total / BM + p.B : p.B * ((p.L + BM - 1) / BM)) * p.H;
     const int64_t round = 8 * XCD_GROUP;                 // the id regrouping is a bijection on multiples of this
     const int nblocks = int((tiles + round - 1) / round * round);
@@ -883,20 +912,26 @@ hipError_t tdb_launch_mfma(const TdbKernelParams& p, int, hipStream_t stream) {
     const dim3 grid(unsigned(p.varlen ? nblocks : persistent)), block(NTHREADS);
     const size_t smem = sizeof(Smem);
     const bool c2p = p.pk != nullptr, p2c = p.pq != nullptr;
-#define TDB_LAUNCH(A, B)                                                                                        \
+#define TDB_LAUNCH(A, B, T)                                                                                     \
     do {                                                                                                        \
         static bool attr_set = false;                                                                           \
         if (!attr_set) {                                                                                        \
-            hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_mfma_kernel<A, B>),                         \
-                                hipFuncAttributeMaxDynamicSharedMemorySize, int(smem));                         \
+            (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_mfma_kernel<A, B, T>),                \
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, int(smem));                   \
             attr_set = true;                                                                                    \
         }                                                                                                       \
-        hipLaunchKernelGGL((attn_mfma_kernel<A, B>), grid, block, smem, stream, p, nblocks);                        \
+        hipLaunchKernelGGL((attn_mfma_kernel<A, B, T>), grid, block, smem, stream, p, nblocks);                 \
     } while (0)
-    if (c2p && p2c) TDB_LAUNCH(true, true);
-    else if (c2p) TDB_LAUNCH(true, false);
-    else if (p2c) TDB_LAUNCH(false, true);
-    else TDB_LAUNCH(false, false);
+#define TDB_LAUNCH_T(T)                                                                                         \
+    do {                                                                                                        \
+        if (c2p && p2c) TDB_LAUNCH(true, true, T);                                                              \
+        else if (c2p) TDB_LAUNCH(true, false, T);                                                               \
+        else if (p2c) TDB_LAUNCH(false, true, T);                                                               \
+        else TDB_LAUNCH(false, false, T);                                                                       \
+    } while (0)
+    if (dtype == TDB_F16) TDB_LAUNCH_T(TDB_F16);
+    else TDB_LAUNCH_T(TDB_BF16);
+#undef TDB_LAUNCH_T
 #undef TDB_LAUNCH
     return hipGetLastError();
 }
