@@ -168,8 +168,9 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     auto delta_of = [&](int r) { return p.lut[min(max(r + p.lut_half, 0), lut_max)]; };
 
     struct Tile {
-        int vb, head, b, row0, len;
+        int vb, head, b, row0, len;       // vb < 0: no tile
         int64_t tok0;
+        int cost;                         // balanced walk: cost coordinate of the tile (see below)
     };
     auto tile_index = [&](int vb, int& hd, int& tile_id) {   // false: the virtual block has no tile
         const int xcd = vb & 7, slot = vb >> 3;
@@ -233,13 +234,86 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         }
         return false;
     };
+    // Packed launches of up to 64 sequences use a cost-balanced walk instead of the strided one: tiles differ in
+    // length by up to 8x, so workgroup g takes a CONTIGUOUS range of the tile list (heads outermost, then sequences,
+    // then the query tiles of a sequence) whose summed cost is 1/gridDim.x of the total.  The cost of a tile is
+    // 8 * (its key steps) + 13, in eighths of a key step (13: what opening a tile costs).  Every wave derives the
+    // same ranges from the boundaries in its lanes; a tile belongs to the workgroup whose cost interval holds the
+    // tile's start coordinate.  Consecutive query tiles of a sequence then run back to back on one CU.
+    const bool balanced = p.varlen && p.B <= 64;
+    int n_lane = 0, pre_lane = 0, cost_per_head = 0, cost_end = 0;
+    auto tiles_of = [](int n) { return (n + BM - 1) / BM; };
+    auto cost_of = [](int n) { return 8 * ((n + BN - 1) / BN) + 13; };
+    if (balanced) {
+        if (l < p.B) {
+            n_lane = cu_hi - cu_lo;
+            if (cu_lo < 0 || n_lane < 0 || cu_hi > p.total) n_lane = 0;   // malformed entry: no tiles
+            n_lane = min(n_lane, p.L);
+        }
+        pre_lane = tiles_of(n_lane) * cost_of(n_lane);                    // inclusive prefix sum over the wave
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const int up = __shfl_up(pre_lane, d);
+            if (l >= d) pre_lane += up;
+        }
+        cost_per_head = __builtin_amdgcn_readlane(pre_lane, 63);
+    }
+    // Moves (head, sequence, tile) forward until it names an existing tile; t.cost is its start coordinate.
+    auto settle = [&](Tile t, int tile_in_seq) {
+        const unsigned long long have = __builtin_amdgcn_ballot_w64(n_lane > 0);
+        while (t.head < p.H) {
+            const int n = __builtin_amdgcn_readlane(n_lane, t.b);
+            if (tile_in_seq < tiles_of(n)) {
+                t.row0 = tile_in_seq * BM;
+                t.len = n;
+                t.tok0 = __builtin_amdgcn_readlane(cu_lo, t.b);
+                t.vb = t.cost < cost_end ? 0 : -1;
+                return t;
+            }
+            const unsigned long long later = t.b >= 63 ? 0ull : have & ~((2ull << t.b) - 1ull);
+            tile_in_seq = 0;
+            if (later) {
+                t.b = __builtin_ctzll(later);
+            } else {                      // next head (a launch without any tile never gets here: cost_per_head > 0)
+                t.head += 1;
+                t.b = __builtin_ctzll(have);
+                t.cost = t.head * cost_per_head;
+            }
+        }
+        t.vb = -1;
+        return t;
+    };
+    auto first_balanced = [&]() {
+        Tile t;
+        t.vb = -1;
+        t.head = t.b = t.row0 = t.len = t.cost = 0;
+        t.tok0 = 0;
+        if (cost_per_head <= 0) return t;
+        const int64_t total = int64_t(cost_per_head) * p.H;
+        const int start = int(total * blockIdx.x / gridDim.x);
+        cost_end = int(total * (blockIdx.x + 1) / gridDim.x);
+        t.head = start / cost_per_head;
+        const int rem = start - t.head * cost_per_head;
+        const unsigned long long owners = __builtin_amdgcn_ballot_w64(pre_lane > rem);
+        t.b = __builtin_amdgcn_readfirstlane(__builtin_ctzll(owners));
+        const int n = __builtin_amdgcn_readlane(n_lane, t.b);
+        const int before = __builtin_amdgcn_readlane(pre_lane, t.b) - tiles_of(n) * cost_of(n);
+        const int tile_in_seq = (rem - before + cost_of(n) - 1) / cost_of(n);     // first tile starting at or after rem
+        t.cost = t.head * cost_per_head + before + tile_in_seq * cost_of(n);
+        return settle(t, tile_in_seq);
+    };
+    auto next_balanced = [&](Tile t) {
+        if (t.vb < 0) return t;
+        t.cost += cost_of(t.len);
+        return settle(t, t.row0 / BM + 1);
+    };
     // First tile with live query rows among the virtual blocks vb, vb + gridDim.x, ...; vb = -1 if there is none.
     // Tiles that hold only padded query rows (fixed layout) get their zeros here, from whoever looks them up:
     // every wave of the workgroup walks the same list, each thread fills its share.
     auto find_tile = [&](int vb) {
         Tile t;
         t.vb = -1;
-        t.head = t.b = t.row0 = t.len = 0;
+        t.head = t.b = t.row0 = t.len = t.cost = 0;
         t.tok0 = 0;
         for (; vb < nblocks; vb += gridDim.x) {
             int hd, tile_id;
@@ -270,7 +344,9 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     auto pk_of = [&](const Tile& t) { return HAS_C2P ? static_cast<const uint16_t*>(p.pk) + int64_t(t.head) * p.pks_h : nullptr; };
     auto pq_of = [&](const Tile& t) { return HAS_P2C ? static_cast<const uint16_t*>(p.pq) + int64_t(t.head) * p.pqs_h : nullptr; };
 
-    Tile cur = find_tile(blockIdx.x);
+    auto next_tile = [&](const Tile& t) { return balanced ? next_balanced(t) : find_tile(t.vb + gridDim.x); };
+
+    Tile cur = balanced ? first_balanced() : find_tile(blockIdx.x);
     if (cur.vb < 0) return;
 
     // ---- pipeline of one tile -----------------------------------------------------------------------------------
@@ -560,7 +636,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
             // to LDS in half A of the last step, where this role has nothing else to do: after the barrier that ends
             // that half, it is already at the next tile's first position products while the score waves finish the
             // last step.
-            const Tile nxt = find_tile(cur.vb + gridDim.x);
+            const Tile nxt = next_tile(cur);
             TDB_PSTAMP(7);
 
             int off2 = prev_off(off1);    // ring offset of step s+2
@@ -821,7 +897,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         phase_barrier();
         TDB_PSTAMP(5);
         // the tile after this one is looked up while the position waves get step 1 ready
-        nxt = find_tile(cur.vb + gridDim.x);
+        nxt = next_tile(cur);
         TDB_PSTAMP(1);
         load_q(qb_next, nxt);
         TDB_PSTAMP(2);
@@ -905,11 +981,11 @@ hipError_t tdb_launch_mfma(const TdbKernelParams& p, int dtype, hipStream_t stre
         if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 8) n = 8;
         cus_of[dev] = n / 8 * 8;
     }
-    // Fixed layout: persistent workgroups, one per CU (tiles cost the same, a static deal is balanced).  Packed:
-    // tiles differ in length by up to 8x, so every tile gets its own workgroup and the hardware dispatcher hands
-    // them to CUs as they free up.
+    // Persistent workgroups, one per CU: fixed layout with a strided deal (tiles cost about the same), packed
+    // batches of up to 64 sequences with a cost-balanced deal computed in the kernel.  Larger packed batches: every
+    // tile gets its own workgroup and the hardware dispatcher hands them to CUs as they free up.
     const int persistent = nblocks < cus_of[dev] ? nblocks : cus_of[dev];
-    const dim3 grid(unsigned(p.varlen ? nblocks : persistent)), block(NTHREADS);
+    const dim3 grid(unsigned(p.varlen && p.B > 64 ? nblocks : persistent)), block(NTHREADS);
     const size_t smem = sizeof(Smem);
     const bool c2p = p.pk != nullptr, p2c = p.pq != nullptr;
 #define TDB_LAUNCH(A, B, T)                                                                                     \
