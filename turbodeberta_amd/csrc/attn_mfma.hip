@@ -549,7 +549,6 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         // the 64 new rows of steps 1 to 3), the row reads depend on them.
         int dl_win[WIN / 32], dl_step[3][2];
         u32x4 st_k[4], st_wk[WIN / 32], st_wq[WIN / 32];
-        X8 qb_next[4];
         // (Both readers assign every register also when there is no next tile: a conditional assignment would keep the
         // previous tile's values alive across the whole tile body.)
         auto read_deltas = [&](const Tile& t) {
@@ -675,7 +674,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
             phase_barrier();
             TDB_STAMP(0);
             read_stage(nxt);
-            load_q(qb_next, nxt);
+            load_q(qb, nxt);              // (the last products of this tile have read the old fragments)
             if (nxt.vb >= 0) write_stage();
             TDB_STAMP(1);
             phase_barrier();
@@ -683,8 +682,6 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
             if (nxt.vb < 0) break;
             cur = nxt;
             bind(cur);
-#pragma unroll
-            for (int c = 0; c < 4; ++c) qb[c] = qb_next[c];
         }
         TDB_T_FLUSH(6);
         TDB_P_FLUSH;
@@ -736,6 +733,10 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
             *reinterpret_cast<u32x4*>(&sm.v[(srow + 32 * n) * RS + sch * 8]) = pre_v[n];
         }
     };
+    Tile nxt;                             // the tile after the current one (looked up while a tile opens)
+    nxt.vb = -1;
+    nxt.head = nxt.b = nxt.row0 = nxt.len = nxt.cost = 0;
+    nxt.tok0 = 0;
     TDB_T_DECL
     // One key step.  MASKED: the step reaches past the end of the sequence (only the last step can).
     auto key_step = [&](int s, auto masked_tag) {
@@ -797,6 +798,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
 #pragma unroll
             for (int jt = 0; jt < 2; ++jt) s_acc[jt] = E::mfma(kf[jt][c], qb[c], s_acc[jt]);
         load_kf((s + 1) & 1);             // K fragments of step s+1 (the MFMAs above have read this step's)
+        if (s + 1 == nsteps) load_q(qb, nxt);   // last step: the Q fragments of the next tile travel from here on
         if (s + 1 < nsteps) fetch_kv(s + 3, s + 1);   // for the next half A (nothing left to fetch in the last step)
         // V^T fragments through the transposing LDS read: the lane provides the address of 4 dims of one key
         X8 vf[2][2][2];               // [key tile][16-key chunk][dim tile]
@@ -871,12 +873,9 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     };
 
     // Opening of a tile, after its first barrier (first stage in LDS).  Everything that reads global memory is
-    // requested here and waited for much later: keys of step 2 / values of step 0 (stored in half A of step 0) and
-    // the Q fragments of the tile after this one.  The output rows of the previous tile are written
+    // requested here and waited for much later: keys of step 2 / values of step 0 (stored in half A of step 0).  The output rows of the previous tile are written
     // last: stores count on the same in-order counter as loads, so a wait for any load issued after them would
     // also wait for them.
-    Tile nxt;
-    X8 qb_next[4];
     u32x2 o_out[2][4];                    // packed output rows of the tile just finished
     uint16_t* o_ptr = nullptr;
     bool o_write = false;
@@ -899,8 +898,6 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         // the tile after this one is looked up while the position waves get step 1 ready
         nxt = next_tile(cur);
         TDB_PSTAMP(1);
-        load_q(qb_next, nxt);
-        TDB_PSTAMP(2);
     };
     // epilogue of a tile: normalised output rows, packed; lane holds d = 32*dt + 8*a + 4*hh + 0..3 of query row il
     auto close_tile = [&]() {
@@ -939,8 +936,6 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         if (nxt.vb < 0) break;
         cur = nxt;
         bind(cur);
-#pragma unroll
-        for (int c = 0; c < 4; ++c) qb[c] = qb_next[c];
         open_tile();
     }
     if (o_write) {
