@@ -876,7 +876,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     // requested here and waited for much later: keys of step 2 / values of step 0 (stored in half A of step 0).  The output rows of the previous tile are written
     // last: stores count on the same in-order counter as loads, so a wait for any load issued after them would
     // also wait for them.
-    u32x2 o_out[2][4];                    // packed output rows of the tile just finished
+    u32x4 o_out[2][2];                    // packed output rows of the tile just finished, 16 B per store
     uint16_t* o_ptr = nullptr;
     bool o_write = false;
     auto open_tile = [&]() {
@@ -888,7 +888,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
 #pragma unroll
             for (int dt = 0; dt < 2; ++dt)
 #pragma unroll
-                for (int a = 0; a < 4; ++a) *reinterpret_cast<u32x2*>(o_ptr + 32 * dt + 8 * a) = o_out[dt][a];
+                for (int a = 0; a < 2; ++a) *reinterpret_cast<u32x4*>(o_ptr + 32 * dt + 16 * a) = o_out[dt][a];
         }
         TDB_PSTAMP(3);
         phase_barrier();                  // the two opening barriers of the position waves
@@ -899,21 +899,31 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         nxt = next_tile(cur);
         TDB_PSTAMP(1);
     };
-    // epilogue of a tile: normalised output rows, packed; lane holds d = 32*dt + 8*a + 4*hh + 0..3 of query row il
+    // Epilogue of a tile: normalised output rows, packed.  A lane holds d = 32*dt + 8*a + 4*hh + 0..3 of query row il,
+    // its partner lane^32 the other four of every eight; one swap between the lane halves per dword gives each lane
+    // eight consecutive d (lane half hh keeps the blocks a = 2*a2 + hh), so a row goes out in 16-byte stores.
     auto close_tile = [&]() {
         const int qi = row0 + 32 * w + il;
         const float l_tot = l_run + __shfl_xor(l_run, 32);
         const float inv = 1.f / l_tot;
         const bool live = qi < len;
         o_write = qi < row0 + rows_here;
-        o_ptr = O + int64_t(qi) * p.os_l + 4 * hh;
+        o_ptr = O + int64_t(qi) * p.os_l + 8 * hh;
 #pragma unroll
         for (int dt = 0; dt < 2; ++dt)
 #pragma unroll
-            for (int a = 0; a < 4; ++a) {
-                u32x2 r = {0, 0};
-                if (live) r = pack4<E>(o_acc[dt][4 * a] * inv, o_acc[dt][4 * a + 1] * inv, o_acc[dt][4 * a + 2] * inv, o_acc[dt][4 * a + 3] * inv);
-                o_out[dt][a] = r;
+            for (int a2 = 0; a2 < 2; ++a2) {
+                u32x2 r[2];
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    const int a = 2 * a2 + t;
+                    r[t] = u32x2{0, 0};
+                    if (live) r[t] = pack4<E>(o_acc[dt][4 * a] * inv, o_acc[dt][4 * a + 1] * inv, o_acc[dt][4 * a + 2] * inv, o_acc[dt][4 * a + 3] * inv);
+                }
+                // lower half: (own block 2*a2, partner's block 2*a2); upper half: (partner's block 2*a2+1, own block 2*a2+1)
+                const auto k0 = __builtin_amdgcn_permlane32_swap(r[0][0], r[1][0], false, false);
+                const auto k1 = __builtin_amdgcn_permlane32_swap(r[0][1], r[1][1], false, false);
+                o_out[dt][a2] = u32x4{k0[0], k1[0], k0[1], k1[1]};
             }
     };
 
@@ -942,7 +952,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
 #pragma unroll
         for (int dt = 0; dt < 2; ++dt)
 #pragma unroll
-            for (int a = 0; a < 4; ++a) *reinterpret_cast<u32x2*>(o_ptr + 32 * dt + 8 * a) = o_out[dt][a];
+            for (int a = 0; a < 2; ++a) *reinterpret_cast<u32x4*>(o_ptr + 32 * dt + 16 * a) = o_out[dt][a];
     }
     TDB_T_FLUSH(0);
     TDB_P_FLUSH;
