@@ -148,7 +148,8 @@ def model_benchmark(dev, steps=10, warmup=3):
     """End-to-end forward of a DeBERTa-v3-large-shaped model (24 layers x 1024, 16 heads x 64, FFN 4096, vocabulary
     128100, buckets 256, max_rel 512, shared keys, c2p|p2c, layer-normed relative embeddings; random N(0, 0.02)
     weights, eval mode, bf16) on ids [16, 512] with right-padded lengths U[64, 512]: valid tokens per second with the
-    attention core on the fused kernel, and with Hugging Face's eager attention in the same model on the same GPU."""
+    attention core on the fused kernel (encoder packed: the default; and with padded layers), and with Hugging Face's
+    eager attention in the same model on the same GPU."""
     from transformers import DebertaV2Config, DebertaV2Model
     from turbodeberta_amd.model import patch_model
     cfg = DebertaV2Config(vocab_size=128100, hidden_size=1024, num_hidden_layers=24, num_attention_heads=16,
@@ -178,11 +179,17 @@ def model_benchmark(dev, steps=10, warmup=3):
         return (time.perf_counter() - t0) / steps
 
     t_eager = run(model)
-    t_fused = run(patch_model(model))
+    patch_model(model)
+    model.encoder.pack_sequences = False
+    t_padded = run(model)
+    model.encoder.pack_sequences = True
+    t_fused = run(model)
     tokens = float(lengths.sum())
     return {"workload": "v3-large-shaped model, ids [16, 512], lengths U[64,512] seed 0 (%d valid tokens), bf16" % int(tokens),
             "steps": steps, "warmup": warmup,
             "fused": {"ms_per_forward": round(t_fused * 1e3, 3), "valid_tokens_per_s": round(tokens / t_fused, 1)},
+            "fused_padded_layers": {"ms_per_forward": round(t_padded * 1e3, 3),
+                                    "valid_tokens_per_s": round(tokens / t_padded, 1)},
             "hf_eager_same_gpu": {"ms_per_forward": round(t_eager * 1e3, 3), "valid_tokens_per_s": round(tokens / t_eager, 1)},
             "speedup": round(t_eager / t_fused, 3)}
 

@@ -180,3 +180,69 @@ def test_eval_caches_follow_weight_updates():
     b = model(input_ids=ids, attention_mask=mask2).last_hidden_state.detach()
     v2 = mask2.bool()
     assert (a[v2] - b[v2]).abs().max() <= 1e-5 * b[v2].abs().max()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("conv", [0, 3])
+def test_packed_encoder_matches_hf_eager_and_padded_path(conv):
+    """Eval mode keeps a batch with padding packed through the whole encoder.  fp32, 3 layers (with and without the
+    convolution after the first layer): against Hugging Face's eager model on the same device, against the padded
+    path of the same model, every layer's output when asked for, zeros at padded positions, and an unpadded batch."""
+    cfg = DebertaV2Config(**dict(tiny_model_config(), num_hidden_layers=3, conv_kernel_size=conv, conv_act="gelu"))
+    theirs = DebertaV2Model(cfg).eval()
+    fill_params(theirs, seed=11)
+    ours = FlashDebertaV2Model(cfg).eval()
+    ours.load_state_dict(theirs.state_dict())
+    ours, theirs = ours.to("cuda:0"), theirs.to("cuda:0")
+    rs = np.random.RandomState(3)
+    B, L = 5, 40
+    lens = np.array([40, 1, 17, 33, 8])
+    ids = torch.from_numpy(rs.randint(1, cfg.vocab_size, size=(B, L))).cuda()
+    mask = torch.from_numpy((np.arange(L)[None] < lens[:, None]).astype(np.int64)).cuda()
+    valid = mask.bool()
+    print(f"[case] packed encoder conv={conv}", flush=True)
+    with torch.no_grad():
+        want = theirs(input_ids=ids, attention_mask=mask, output_hidden_states=True)
+        got = ours(input_ids=ids, attention_mask=mask, output_hidden_states=True)
+        ours.encoder.pack_sequences = False
+        padded = ours(input_ids=ids, attention_mask=mask, output_hidden_states=True)
+        ours.encoder.pack_sequences = True
+        last_only = ours(input_ids=ids, attention_mask=mask)
+    assert len(got.hidden_states) == len(want.hidden_states) == 4
+    for g, p, w in zip(got.hidden_states, padded.hidden_states, want.hidden_states):
+        scale = w[valid].abs().max().item()
+        assert (g[valid] - w[valid]).abs().max().item() <= 1e-4 * scale
+        assert (g[valid] - p[valid]).abs().max().item() <= 1e-5 * scale
+    assert bool(torch.equal(got.last_hidden_state, got.hidden_states[-1]))
+    assert got.last_hidden_state[~valid].abs().max().item() == 0.0
+    assert last_only.hidden_states is None
+    # (the library convolution may pick another algorithm on a later call: equal to rounding, not to the bit)
+    assert (last_only.last_hidden_state - got.last_hidden_state).abs().max().item() <= 1e-5 * scale
+    # a batch without padding takes the padded path (nothing to pack) and still agrees
+    full = torch.ones_like(mask)
+    with torch.no_grad():
+        a = ours(input_ids=ids, attention_mask=full).last_hidden_state
+        b = theirs(input_ids=ids, attention_mask=full).last_hidden_state
+    assert (a - b).abs().max().item() <= 1e-4 * b.abs().max().item()
+
+
+@pytest.mark.gpu
+def test_patch_model_packs_a_task_head():
+    """``patch_model`` on a Hugging Face task model: the encoder inside runs packed, logits equal eager's."""
+    from transformers.models.deberta_v2.modeling_deberta_v2 import DebertaV2ForTokenClassification
+    from turbodeberta_amd.model import FlashDebertaV2Encoder
+    cfg = DebertaV2Config(**dict(tiny_model_config(), num_labels=5))
+    theirs = DebertaV2ForTokenClassification(cfg).eval()
+    fill_params(theirs, seed=2)
+    ours = DebertaV2ForTokenClassification(cfg).eval()
+    ours.load_state_dict(theirs.state_dict())
+    assert isinstance(patch_model(ours).deberta.encoder, FlashDebertaV2Encoder)
+    ours, theirs = ours.to("cuda:0"), theirs.to("cuda:0")
+    ids, mask = tiny_model_inputs()
+    ids, mask = torch.from_numpy(ids).cuda(), torch.from_numpy(mask).cuda()
+    print("[case] patched token classifier", flush=True)
+    with torch.no_grad():
+        a = ours(input_ids=ids, attention_mask=mask).logits
+        b = theirs(input_ids=ids, attention_mask=mask).logits
+    valid = mask.bool()
+    assert (a[valid] - b[valid]).abs().max().item() <= 1e-4 * b[valid].abs().max().item()

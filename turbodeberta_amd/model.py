@@ -19,7 +19,13 @@ What differs from the reference glue (model.py:34-186):
   only; the reference recomputes both strip GEMMs every call, model.py:94-110) and the
   concatenated Q/K/V weight of the single fused projection GEMM; the valid lengths are computed by
   the first layer that sees a mask and reused by the others (the reference recomputes them, with
-  a host synchronisation, in every layer: model.py:55-63).
+  a host synchronisation, in every layer: model.py:55-63);
+* in eval mode the encoder keeps a batch with padding packed from the embeddings to the last layer:
+  projections, LayerNorms and feed-forward blocks run on ``[valid_tokens, hidden]`` and the packed
+  attention kernel is called with views of the projection output, so padded positions cost
+  nothing anywhere.  The reference packs and re-pads around the attention call of every layer
+  (model.py:138-183); here there is one gather after the embeddings, one scatter at the end and one
+  host synchronisation (the number of valid tokens) per forward.
 """
 from __future__ import annotations
 
@@ -28,6 +34,7 @@ from typing import Optional
 
 import torch
 from torch import nn
+from transformers.modeling_outputs import BaseModelOutput
 from transformers.models.deberta_v2.modeling_deberta_v2 import (
     DebertaV2Attention,
     DebertaV2Encoder,
@@ -37,7 +44,8 @@ from transformers.models.deberta_v2.modeling_deberta_v2 import (
 )
 
 from .ops.flash_attention import flash_attention_with_disentangled
-from .padding import key_padding_mask
+from .ops.flash_attention_varlen import flash_attention_with_disentangled_varlen
+from .padding import _get_unpad_data, index_first_axis, key_padding_mask, pad_input
 
 
 def _versions(*tensors):
@@ -95,26 +103,43 @@ class FlashDisentangledSelfAttention(DisentangledSelfAttention):
             k = heads(self.key_proj(hidden_states))
             v = heads(self.value_proj(hidden_states))
 
-        scale_factor = 1 + int("c2p" in self.pos_att_type) + int("p2c" in self.pos_att_type)
-        pos_key = pos_query = None
-        buckets = max_rel = 0
-        if self.relative_attention:
-            buckets, max_rel = self.position_buckets, self.max_relative_positions
-            span = self.pos_ebd_size
-            if frozen:
-                pos_key, pos_query = self._position_tables(rel_embeddings, hidden_states.dtype)
-            else:
-                pos_key, pos_query = self._project_tables(self.pos_dropout(rel_embeddings)[0:2 * span])   # HF:295
-        else:
-            scale_factor = 1
-        sm_scale = 1.0 / math.sqrt(D * scale_factor)                                             # HF:120-121, :243
-
+        pos_key, pos_query, sm_scale, buckets, max_rel = self._position_terms(rel_embeddings, hidden_states.dtype,
+                                                                              frozen)
         seqlens = _lengths_of(attention_mask) if attention_mask is not None else None
         out = flash_attention_with_disentangled(q, k, v, None, None, False, sm_scale, buckets, max_rel,
                                                 pos_key_layer=pos_key, pos_query_layer=pos_query,
                                                 seqlens_k=seqlens)
         # out has q's strides: [B, H, L, D] view of token-major storage
         return (out.permute(0, 2, 1, 3).reshape(B, L, H * D), None)
+
+    def forward_packed(self, hidden_states, cu_seqlens, max_seqlen, rel_embeddings=None):
+        """Eval-mode forward on packed tokens: ``hidden_states [T, hidden]`` holds the valid tokens of all
+        sequences back to back, ``cu_seqlens`` int32 ``[B+1]`` their boundaries.  Returns ``[T, H*D]``.
+        The counterpart of the reference's packed branch (model.py:138-183) without its per-layer gathers."""
+        T = hidden_states.shape[0]
+        H, D = self.num_attention_heads, self.attention_head_size
+        w, b = self._fused_qkv()
+        qkv = nn.functional.linear(hidden_states, w, b).view(T, 3, H, D)
+        pos_key, pos_query, sm_scale, buckets, max_rel = self._position_terms(rel_embeddings, hidden_states.dtype, True)
+        out = flash_attention_with_disentangled_varlen(qkv[:, 0], qkv[:, 1], qkv[:, 2], None, None, cu_seqlens,
+                                                       cu_seqlens, max_seqlen, max_seqlen, False, sm_scale, buckets,
+                                                       max_rel, pos_key_layer=pos_key, pos_query_layer=pos_query)
+        return out.reshape(T, H * D)
+
+    def _position_terms(self, rel_embeddings, dtype, frozen):
+        """``(pos_key, pos_query, sm_scale, position_buckets, max_relative_positions)`` of one call."""
+        scale_factor = 1
+        pos_key = pos_query = None
+        buckets = max_rel = 0
+        if self.relative_attention:
+            scale_factor += int("c2p" in self.pos_att_type) + int("p2c" in self.pos_att_type)
+            buckets, max_rel = self.position_buckets, self.max_relative_positions
+            if frozen:
+                pos_key, pos_query = self._position_tables(rel_embeddings, dtype)
+            else:
+                rel = self.pos_dropout(rel_embeddings)[0:2 * self.pos_ebd_size]                 # HF:295
+                pos_key, pos_query = self._project_tables(rel)
+        return pos_key, pos_query, 1.0 / math.sqrt(self.attention_head_size * scale_factor), buckets, max_rel   # HF:120-121, :243
 
     def _project_tables(self, rel):
         """Per-head projections of the relative embeddings, ``[H, 2*span, D]`` views (modeling_deberta_v2.py:296-312)."""
@@ -168,9 +193,61 @@ class FlashDebertaV2Layer(DebertaV2Layer):
 
 
 class FlashDebertaV2Encoder(DebertaV2Encoder):
+    """``DebertaV2Encoder`` (modeling_deberta_v2.py:565-686) over ``FlashDebertaV2Layer``.
+
+    In eval mode under ``torch.no_grad()`` a batch that contains padding runs **packed**: the valid tokens
+    are gathered once, every layer works on ``[valid_tokens, hidden]`` (``forward_packed`` of the attention
+    module, then Hugging Face's own output / feed-forward submodules, which are shape agnostic), and the
+    result is scattered back to ``[B, L, hidden]`` with zeros at padded positions.  Counting the valid
+    tokens is the only host synchronisation of the forward.  Everything else -- training, gradients,
+    ``output_attentions``, ``query_states``, masks that are not ``[B, L]``-reducible, CPU tensors, batches
+    without padding -- takes the parent's loop over the (fused, padded) layers.
+
+    ``pack_sequences = False`` switches the packed path off."""
+
+    pack_sequences = True
+    _tdb_all_hidden = True      # cleared by FlashDebertaV2Model when the caller did not ask for every layer's output
+
     def __init__(self, config):
         super().__init__(config)
         self.layer = nn.ModuleList([FlashDebertaV2Layer(config) for _ in range(config.num_hidden_layers)])
+
+    def forward(self, hidden_states, attention_mask, output_hidden_states=True, output_attentions=False,
+                query_states=None, relative_pos=None, return_dict=True):
+        fused = (not output_attentions and torch.is_tensor(hidden_states)
+                 and all(isinstance(l.attention.self, FlashDisentangledSelfAttention) for l in self.layer))
+        packable = (fused and self.pack_sequences and not self.training and not torch.is_grad_enabled()
+                    and query_states is None and hidden_states.is_cuda and attention_mask.dim() in (2, 3, 4))
+        if packable:
+            B, L, _ = hidden_states.shape
+            indices, cu_seqlens, _ = _get_unpad_data(attention_mask)       # the one host synchronisation
+            packable = indices.numel() < B * L
+        if not packable:
+            if fused and relative_pos is None and self.relative_attention:
+                relative_pos = hidden_states.new_empty(0)    # fused layers never read the [L, L] matrix: do not build it
+            return super().forward(hidden_states, attention_mask, output_hidden_states, output_attentions,
+                                   query_states, relative_pos, return_dict)
+
+        keep_all = output_hidden_states and self._tdb_all_hidden
+        padded = lambda t: pad_input(t, indices, B, L)
+        all_hidden_states = (hidden_states,) if output_hidden_states else None
+        rel_embeddings = self.get_rel_embedding()
+        x = index_first_axis(hidden_states.reshape(B * L, -1), indices)
+        for i, layer in enumerate(self.layer):
+            attn = layer.attention
+            attended = attn.output(attn.self.forward_packed(x, cu_seqlens, L, rel_embeddings), x)     # HF:368-378
+            x = layer.output(layer.intermediate(attended), attended)                                   # HF:431-432
+            if i == 0 and self.conv is not None:                                                       # HF:666-667
+                x = index_first_axis(self.conv(hidden_states, padded(x), key_padding_mask(attention_mask).long())
+                                     .reshape(B * L, -1), indices)
+            if keep_all and i + 1 < len(self.layer):
+                all_hidden_states = all_hidden_states + (padded(x),)
+        output_states = padded(x)
+        if output_hidden_states:
+            all_hidden_states = all_hidden_states + (output_states,)
+        if not return_dict:
+            return tuple(v for v in [output_states, all_hidden_states, None] if v is not None)
+        return BaseModelOutput(last_hidden_state=output_states, hidden_states=all_hidden_states, attentions=None)
 
 
 class FlashDebertaV2Model(DebertaV2Model):
@@ -179,11 +256,28 @@ class FlashDebertaV2Model(DebertaV2Model):
         self.encoder = FlashDebertaV2Encoder(config)
         self.post_init()
 
+    def forward(self, input_ids=None, attention_mask=None, token_type_ids=None, position_ids=None,
+                inputs_embeds=None, output_attentions=None, output_hidden_states=None, return_dict=None, **kwargs):
+        # The parent always asks the encoder for every layer's output and then uses the last one
+        # (modeling_deberta_v2.py:760-768); tell the packed encoder whether the caller wants the others too,
+        # so that it does not scatter 24 intermediate results back to [B, L, hidden] for nothing.
+        wanted = output_hidden_states if output_hidden_states is not None else self.config.output_hidden_states
+        self.encoder._tdb_all_hidden = bool(wanted) or self.z_steps > 1
+        try:
+            return super().forward(input_ids=input_ids, attention_mask=attention_mask, token_type_ids=token_type_ids,
+                                   position_ids=position_ids, inputs_embeds=inputs_embeds,
+                                   output_attentions=output_attentions, output_hidden_states=output_hidden_states,
+                                   return_dict=return_dict, **kwargs)
+        finally:
+            self.encoder._tdb_all_hidden = True
+
 
 def patch_model(model: nn.Module) -> nn.Module:
     """Switch every ``DisentangledSelfAttention`` inside ``model`` (any DeBERTa-v2/v3 model or task head,
     e.g. one loaded with ``from_pretrained``) to the fused kernel, in place.  Parameters are untouched."""
+    swaps = {DisentangledSelfAttention: FlashDisentangledSelfAttention, DebertaV2Encoder: FlashDebertaV2Encoder,
+             DebertaV2Model: FlashDebertaV2Model}        # none of them adds parameters or constructor state
     for module in model.modules():
-        if type(module) is DisentangledSelfAttention:
-            module.__class__ = FlashDisentangledSelfAttention
+        if type(module) in swaps:
+            module.__class__ = swaps[type(module)]
     return model
