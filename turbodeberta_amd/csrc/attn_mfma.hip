@@ -60,8 +60,9 @@ struct Smem {
     uint16_t p[BN * PS];
 };
 
-// The two 16-bit element types the kernel is instantiated for: what differs is the MFMA, the dot-product
-// instruction and the float conversion.  (bf16: fp32's range, 8 significant bits; fp16: 11 bits, range 65504 --
+// The two 16-bit element types the kernel is instantiated for: what differs is the MFMA and the float conversion.
+// (No dot-product instructions anywhere: v_dot2 runs on the matrix pipe and would queue behind the other role's MFMAs,
+// while plain vector instructions run beside them.)  (bf16: fp32's range, 8 significant bits; fp16: 11 bits, range 65504 --
 // the p2c products are stored in the element type, the probabilities are at most 2^8.)
 template <int DT>
 struct Elem;
@@ -71,7 +72,11 @@ struct Elem<TDB_BF16> {
     using X2 = bf16x2;
     using X8 = bf16x8;
     static __device__ __forceinline__ f32x16 mfma(X8 a, X8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
-    static __device__ __forceinline__ float dot2(X2 a, X2 b, float c) { return __builtin_amdgcn_fdot2_f32_bf16(a, b, c, false); }
+    // One half of a dword as fp32 through a byte permute (the selector says which half): bf16 -> fp32 is a shift.
+    static constexpr uint32_t PICK_LO = 0x05040c0cu, PICK_HI = 0x07060c0cu;
+    static __device__ __forceinline__ float pick(uint32_t pair, uint32_t sel) {
+        return __builtin_bit_cast(float, __builtin_amdgcn_perm(pair, 0u, sel));
+    }
 };
 template <>
 struct Elem<TDB_F16> {
@@ -79,7 +84,10 @@ struct Elem<TDB_F16> {
     using X2 = f16x2;
     using X8 = f16x8;
     static __device__ __forceinline__ f32x16 mfma(X8 a, X8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
-    static __device__ __forceinline__ float dot2(X2 a, X2 b, float c) { return __builtin_amdgcn_fdot2(a, b, c, false); }
+    static constexpr uint32_t PICK_LO = 0x0c0c0504u, PICK_HI = 0x0c0c0706u;
+    static __device__ __forceinline__ float pick(uint32_t pair, uint32_t sel) {
+        return (float)__builtin_bit_cast(X2, __builtin_amdgcn_perm(pair, 0u, sel))[0];
+    }
 };
 
 template <typename X8>
@@ -690,7 +698,6 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
 
     // ===================================================== score waves ============================================
     const float c_exp = p.scale * 1.4426950408889634f;   // softmax in base 2
-    const X2 ones = {(ET)1.0f, (ET)1.0f};
     f32x16 o_acc[2];
     float m_run, l_run;
 
@@ -767,13 +774,11 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
             // Element (key j, query il) is P'[j][X - j], X = 32w + il + 63: from one key to the next the bf16 index moves
             // by PS - 1 (odd), so the element alternates between the low and the high half of its dword with the
             // parity of j, starting from the parity of il.  The dwords of keys j and j + 2 are (PS - 1) dwords apart
-            // (one two-address read); the unwanted half (a neighbouring, finite P' value) is multiplied by zero in
-            // the dot product that adds the wanted half to the score.
+            // (one two-address read); a byte permute with a per-lane selector moves the wanted half into an fp32.
             constexpr int PD = PS - 1;            // dwords between the elements of keys j and j + 2
             const int X = 32 * w + il + 63, pl = X & 1;
             const auto* pbase = TDB_LDS(const uint32_t, sm.p) + (X - pl) / 2 + 2 * hh * PD;   // dword of element (4hh, X - 4hh)
-            const X2 sel_lo = {(ET)1.0f, (ET)0.0f}, sel_hi = {(ET)0.0f, (ET)1.0f};
-            const X2 sel_even = pl ? sel_hi : sel_lo, sel_odd = pl ? sel_lo : sel_hi;
+            const uint32_t sel_even = pl ? E::PICK_HI : E::PICK_LO, sel_odd = pl ? E::PICK_LO : E::PICK_HI;
             uint32_t g[2][16];
 #pragma unroll
             for (int jt = 0; jt < 2; ++jt)
@@ -786,7 +791,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
             for (int jt = 0; jt < 2; ++jt)
 #pragma unroll
                 for (int e = 0; e < 16; ++e)
-                    s_acc[jt][e] = E::dot2(__builtin_bit_cast(X2, g[jt][e]), (e & 1) ? sel_odd : sel_even, s_acc[jt][e]);
+                    s_acc[jt][e] += E::pick(g[jt][e], (e & 1) ? sel_odd : sel_even);
         }
         TDB_STAMP(1);
         phase_barrier();                  // scratch is free again; keys of step s+1 and values of step s are staged
@@ -859,7 +864,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
                     const float p0 = __builtin_amdgcn_exp2f(fmaf(s_acc[jt][8 * c + 2 * h2], c_exp, -mc));
                     const float p1 = __builtin_amdgcn_exp2f(fmaf(s_acc[jt][8 * c + 2 * h2 + 1], c_exp, -mc));
                     const X2 pr = {(ET)p0, (ET)p1};
-                    psum = E::dot2(pr, ones, psum);   // sum of what the MFMA will see
+                    psum += p0 + p1;
                     pw[h2] = __builtin_bit_cast(uint32_t, pr);
                 }
                 const X8 pb = __builtin_bit_cast(X8, u32x4{pw[0], pw[1], pw[2], pw[3]});
