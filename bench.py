@@ -10,8 +10,8 @@ A "step" is one attention forward over one batch of synthetic DeBERTa-v3-base at
 Prints ONE JSON line.  `value` is algorithmic attention TFLOP/s of the fixed workload over the timed
 region; FLOPs per sequence of valid length l and per head:  4*l*l*d (QK^T + PV) + 4*l*W*d (c2p + p2c),
 W = min(2*span, 2*l - 1) -- no credit for padding, window recompute or projections.
-`roofline` prices the kernel's average launch duration (HIP events on the launch stream) against the
-MI355X dense bf16 MFMA peak; `cpu_baseline` times the CPU oracle (eager float32 restatement of
+`roofline` prices the kernel's average launch duration (two HIP events on the launch stream that bracket the timed
+region, divided by the number of launches) against the MI355X dense bf16 MFMA peak; `cpu_baseline` times the CPU oracle (eager float32 restatement of
 Hugging Face's DisentangledSelfAttention) on a bounded sample of the same workload.
 """
 from __future__ import annotations
@@ -37,7 +37,7 @@ METRIC = "attn TFLOP/s + tokens/s, DeBERTa-v3-base b32xL512 bf16, fixed and varl
 # HBM bytes per launch from `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` runs of this script, each counter scaled
 # by what it reads for a plain 512 MiB device copy (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000); the runs and raw counter
 # values are recorded in profiles/attn_mfma_kernel_fixed_b32xL512.md and profiles/attn_mfma_kernel_varlen_64seq.md.
-MEASURED_TRAFFIC_BYTES = {"fixed": 105.7e6, "varlen": 212.3e6}
+MEASURED_TRAFFIC_BYTES = {"fixed": 106.7e6, "varlen": 213.5e6}
 
 
 def flops_of(lengths) -> float:
@@ -100,16 +100,22 @@ def build_varlen(dev, n_seq=64):
 
 
 def time_steps(plan, steps, warmup):
-    """(wall ms per step over exactly `steps` back-to-back launches, mean kernel ms from HIP events)."""
+    """Times exactly `steps` back-to-back launches after `warmup` untimed ones.  Returns
+    (wall ms per step between two synchronisations, kernel ms = span between two HIP events that bracket the same
+    timed region on the launch stream / steps, then median and minimum of per-launch event pairs from a second pass;
+    an event pair around a single launch reads about 3 us more than the launch takes in a back-to-back stream)."""
     for _ in range(warmup):
         plan.launch()
     torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
+    e0.record()
     for _ in range(steps):
         plan.launch()
+    e1.record()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-    # per-launch duration: an event pair around every launch on the launch stream
+    span_ms = e0.elapsed_time(e1) / steps
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
     for a, b in ev:
         a.record()
@@ -117,7 +123,7 @@ def time_steps(plan, steps, warmup):
         b.record()
     torch.cuda.synchronize()
     durs = sorted(a.elapsed_time(b) for a, b in ev)
-    return wall_ms, float(np.mean(durs)), durs[len(durs) // 2], durs[0]
+    return wall_ms, span_ms, durs[len(durs) // 2], durs[0]
 
 
 def cpu_baseline(tensors, lengths, budget_s=12.0):
@@ -198,7 +204,9 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=200,
+                    help="untimed launches before the timed region (the first ~2 ms of load after an idle period run "
+                         "at a lower clock: 200 launches = 20 ms get past that)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--workload", choices=["both", "fixed", "varlen"], default="both")
     ap.add_argument("--with-model", action="store_true",
@@ -238,8 +246,8 @@ def main():
             "core_tflops": round(H * sum(4.0 * int(l) ** 2 * D for l in lengths) / (wall_ms * 1e-3) / 1e12, 2),
             "roofline": {"bound": "mfma", "achieved": round(ach, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                          "frac": round(ach / PEAK_BF16_TFLOPS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(name), "kernel": kernel,
-                         "kernel_ms_mean": round(mean_ms, 4), "kernel_ms_median": round(med_ms, 4),
-                         "kernel_ms_min": round(min_ms, 4), "algorithmic_gflop": round(fl / 1e9, 3), "algorithmic_bytes": algorithmic_bytes(lengths),
+                         "kernel_ms_mean": round(mean_ms, 4), "kernel_ms_pair_median": round(med_ms, 4),
+                         "kernel_ms_pair_min": round(min_ms, 4), "algorithmic_gflop": round(fl / 1e9, 3), "algorithmic_bytes": algorithmic_bytes(lengths),
                          "hbm_gbs_algorithmic": round(algorithmic_bytes(lengths) / (mean_ms * 1e-3) / 1e9, 1)},
         }
 

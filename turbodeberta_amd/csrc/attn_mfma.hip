@@ -112,6 +112,7 @@ __device__ __forceinline__ u32x2 pack4(float a, float b, float c, float d) {
 // wave, summed per pipeline phase, and entry / exit wall-clock times of every workgroup.
 __device__ long long tdb_timing[16];
 __device__ long long tdb_ptiming[16];
+__device__ long long tdb_wtiming[8 * 6];    // the six phase sums of every wave of that workgroup
 __device__ long long tdb_trace[4 * 4096];   // per workgroup: entry, exit (100 MHz wall clock), hardware id, steps
 #define TDB_T_ENTRY const long long t_entry = __builtin_readcyclecounter(); const long long t_wall = wall_clock64(); \
         long long t_pro[8] = {0, 0, 0, 0, 0, 0, 0, 0}; long long t_plast = t_entry;
@@ -121,10 +122,19 @@ __device__ long long tdb_trace[4 * 4096];   // per workgroup: entry, exit (100 M
 #define TDB_P_FLUSH do { if (blockIdx.x == TDB_TIMING && (threadIdx.x & 255) == 0) \
         for (int t_i = 0; t_i < 8; ++t_i) tdb_ptiming[t_i + (threadIdx.x >> 8) * 8] = t_pro[t_i]; } while (0)
 #define TDB_T_DECL long long t_acc[6] = {0, 0, 0, 0, 0, 0}; long long t_last = __builtin_readcyclecounter(); t_acc[4] = t_last - t_entry;
+// (A stamp is a scalar memory read: it drains the wave's LDS queue and costs about 150 cycles.  TDB_TIMING_LIGHT keeps
+// only the stamps right after a barrier: slot 0 = half B + barrier, slot 2 = half A + barrier.)
+#ifdef TDB_TIMING_LIGHT
+#define TDB_STAMP(slot) do { if ((slot) == 0 || (slot) == 2) { __builtin_amdgcn_sched_barrier(0); const long long t_now = __builtin_readcyclecounter(); \
+        t_acc[slot] += t_now - t_last; t_last = t_now; __builtin_amdgcn_sched_barrier(0); } } while (0)
+#else
 #define TDB_STAMP(slot) do { __builtin_amdgcn_sched_barrier(0); const long long t_now = __builtin_readcyclecounter(); \
         t_acc[slot] += t_now - t_last; t_last = t_now; __builtin_amdgcn_sched_barrier(0); } while (0)
+#endif
 #define TDB_T_FLUSH(base) do { if (blockIdx.x == TDB_TIMING && (threadIdx.x & 255) == 0) \
-        for (int t_i = 0; t_i < 6; ++t_i) tdb_timing[(base) + t_i] = t_acc[t_i]; } while (0)
+        for (int t_i = 0; t_i < 6; ++t_i) tdb_timing[(base) + t_i] = t_acc[t_i]; \
+        if (blockIdx.x == TDB_TIMING && (threadIdx.x & 63) == 0) \
+        for (int t_i = 0; t_i < 6; ++t_i) tdb_wtiming[(threadIdx.x >> 6) * 6 + t_i] = t_acc[t_i]; } while (0)
 #define TDB_TRACE_EXIT do { if (threadIdx.x == 0 && blockIdx.x < 4096) { \
         tdb_trace[4 * blockIdx.x] = t_wall; tdb_trace[4 * blockIdx.x + 1] = wall_clock64(); \
         tdb_trace[4 * blockIdx.x + 2] = (long long)__builtin_amdgcn_s_getreg(63492) | ((long long)__builtin_amdgcn_s_getreg((31 << 11) | 20) << 32); \
