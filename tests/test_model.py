@@ -39,6 +39,21 @@ def test_patch_model_in_place():
     assert all(torch.equal(v, before[k]) for k, v in m.state_dict().items())
 
 
+def test_task_heads_have_hugging_face_parameters():
+    import transformers.models.deberta_v2.modeling_deberta_v2 as hf
+    from turbodeberta_amd import model as ours
+    cfg = DebertaV2Config(**dict(tiny_model_config(), num_labels=3))
+    for name in ("ForMaskedLM", "ForSequenceClassification", "ForTokenClassification", "ForQuestionAnswering",
+                 "ForMultipleChoice"):
+        theirs = getattr(hf, "DebertaV2" + name)(cfg)
+        mine = getattr(ours, "FlashDebertaV2" + name)(cfg)
+        assert list(mine.state_dict()) == list(theirs.state_dict()), name
+        mine.load_state_dict(theirs.state_dict(), strict=True)
+        assert isinstance(mine.deberta, FlashDebertaV2Model) and isinstance(mine.deberta.encoder, ours.FlashDebertaV2Encoder)
+        assert sum(isinstance(m, FlashDisentangledSelfAttention) for m in mine.modules()) == 2
+        assert all(type(m) is not DisentangledSelfAttention for m in mine.modules())
+
+
 def test_forward_without_gpu_fails_loudly():
     m = FlashDebertaV2Model(_tiny()).eval()
     ids, mask = tiny_model_inputs()
@@ -227,6 +242,26 @@ def test_packed_encoder_matches_hf_eager_and_padded_path(conv):
 
 
 @pytest.mark.gpu
+def test_sequence_classifier_matches_hf_eager():
+    from transformers.models.deberta_v2.modeling_deberta_v2 import DebertaV2ForSequenceClassification
+    from turbodeberta_amd.model import FlashDebertaV2ForSequenceClassification
+    cfg = DebertaV2Config(**dict(tiny_model_config(), num_labels=4))
+    theirs = DebertaV2ForSequenceClassification(cfg).eval()
+    fill_params(theirs, seed=8)
+    ours = FlashDebertaV2ForSequenceClassification(cfg).eval()
+    ours.load_state_dict(theirs.state_dict())
+    ours, theirs = ours.to("cuda:0"), theirs.to("cuda:0")
+    ids, mask = tiny_model_inputs()
+    ids, mask = torch.from_numpy(ids).cuda(), torch.from_numpy(mask).cuda()
+    print("[case] sequence classifier", flush=True)
+    with torch.no_grad():
+        a = ours(input_ids=ids, attention_mask=mask).logits
+        b = theirs(input_ids=ids, attention_mask=mask).logits
+    assert a.shape == b.shape == (ids.shape[0], 4)
+    assert (a - b).abs().max().item() <= 1e-4 * b.abs().max().item()
+
+
+@pytest.mark.gpu
 def test_patch_model_packs_a_task_head():
     """``patch_model`` on a Hugging Face task model: the encoder inside runs packed, logits equal eager's."""
     from transformers.models.deberta_v2.modeling_deberta_v2 import DebertaV2ForTokenClassification
@@ -246,3 +281,30 @@ def test_patch_model_packs_a_task_head():
         b = theirs(input_ids=ids, attention_mask=mask).logits
     valid = mask.bool()
     assert (a[valid] - b[valid]).abs().max().item() <= 1e-4 * b[valid].abs().max().item()
+
+
+@pytest.mark.gpu
+def test_query_states_from_another_tensor():
+    """The enhanced-mask-decoder call shape (modeling_deberta_v2.py:772-788): queries projected from ``query_states``,
+    keys and values from ``hidden_states``, against the eager module on the device (fp32)."""
+    cfg = _tiny()
+    theirs = DisentangledSelfAttention(cfg).eval()
+    fill_params(theirs, seed=21)
+    ours = FlashDisentangledSelfAttention(cfg).eval()
+    ours.load_state_dict(theirs.state_dict())
+    ours, theirs = ours.to("cuda:0"), theirs.to("cuda:0")
+    g = torch.Generator().manual_seed(4)
+    B, L = 3, 24
+    hidden = torch.randn(B, L, cfg.hidden_size, generator=g).cuda()
+    queries = torch.randn(B, L, cfg.hidden_size, generator=g).cuda()
+    rel = torch.randn(2 * cfg.position_buckets, cfg.hidden_size, generator=g).cuda()
+    lens = torch.tensor([24, 9, 17])
+    mask2 = (torch.arange(L)[None] < lens[:, None]).long().cuda()
+    ext = mask2.unsqueeze(1).unsqueeze(2)
+    mask4 = ext * ext.squeeze(-2).unsqueeze(-1)
+    print("[case] query_states", flush=True)
+    with torch.no_grad():
+        want = theirs(hidden, mask4, False, query_states=queries, rel_embeddings=rel)[0]
+        got = ours(hidden, mask4, False, query_states=queries, rel_embeddings=rel)[0]
+    valid = mask2.bool()
+    assert (got[valid] - want[valid]).abs().max().item() <= 1e-4 * want[valid].abs().max().item()

@@ -38,6 +38,11 @@ from transformers.modeling_outputs import BaseModelOutput
 from transformers.models.deberta_v2.modeling_deberta_v2 import (
     DebertaV2Attention,
     DebertaV2Encoder,
+    DebertaV2ForMaskedLM,
+    DebertaV2ForMultipleChoice,
+    DebertaV2ForQuestionAnswering,
+    DebertaV2ForSequenceClassification,
+    DebertaV2ForTokenClassification,
     DebertaV2Layer,
     DebertaV2Model,
     DisentangledSelfAttention,
@@ -270,6 +275,38 @@ class FlashDebertaV2Model(DebertaV2Model):
                                    return_dict=return_dict, **kwargs)
         finally:
             self.encoder._tdb_all_hidden = True
+
+
+class _FusedHead:
+    """Task models with the reference's class names (model.py:244-314).  The Hugging Face parent builds the whole
+    model -- so parameter names, weight tying and initialisation are exactly Hugging Face's and stock checkpoints
+    load with ``from_pretrained`` -- and the attention / encoder / model classes inside are then switched to the fused
+    ones.  (The reference's own constructors call ``DebertaV2PreTrainedModel().__init__(config)`` on a fresh,
+    argument-less instance and cannot be instantiated.)"""
+
+    def __init__(self, config):
+        super().__init__(config)
+        patch_model(self)
+
+
+class FlashDebertaV2ForMaskedLM(_FusedHead, DebertaV2ForMaskedLM):
+    pass
+
+
+class FlashDebertaV2ForSequenceClassification(_FusedHead, DebertaV2ForSequenceClassification):
+    pass
+
+
+class FlashDebertaV2ForTokenClassification(_FusedHead, DebertaV2ForTokenClassification):
+    pass
+
+
+class FlashDebertaV2ForQuestionAnswering(_FusedHead, DebertaV2ForQuestionAnswering):
+    pass
+
+
+class FlashDebertaV2ForMultipleChoice(_FusedHead, DebertaV2ForMultipleChoice):
+    pass
 
 
 def patch_model(model: nn.Module) -> nn.Module:
