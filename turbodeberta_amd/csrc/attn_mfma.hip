@@ -501,11 +501,12 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         //   put_results c2p as fp32 C'[i][r'], p2c as bf16 P'[j][r''] into the scratch.
         X8 fr[3][4], fq[2][4], kb[2][4];
         f32x16 res[6];
-        auto load_frags = [&](int o, int kbuf) {
+        auto load_frags = [&](int o, int kbuf, auto first_tag) {
+            constexpr int C_TILES = decltype(first_tag)::value ? 3 : 2;   // (the third tile is carried, see products)
             auto ring = [&](int x) { const int t = x + o; return t >= WIN ? t - WIN : t; };
             if (HAS_C2P) {
 #pragma unroll
-                for (int rt = 0; rt < 3; ++rt) {
+                for (int rt = 0; rt < C_TILES; ++rt) {
                     const int row = ring(32 * w + 32 * rt + il);
 #pragma unroll
                     for (int c = 0; c < 4; ++c) fr[rt][c] = lds_frag<X8>(sm.kr, row, 16 * c + 8 * hh);
@@ -522,7 +523,12 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
                 }
             }
         };
-        auto products = [&]() {
+        // c2p: from one key step to the next the sub-window moves down by 64 positions, so its third tile (positions
+        // 64..95) is the first tile of the step before -- same K_r' rows, same queries, same products.  Only step 0
+        // computes three tiles; later steps compute two and write the carried one (copied to res[2] after it was
+        // written as the first tile) again at its new place.
+        auto products = [&](auto first_tag) {
+            constexpr bool FIRST = decltype(first_tag)::value;
             auto chain = [&](const X8 (&a)[4], const X8 (&bb)[4]) {
                 f32x16 acc = E::mfma(a[0], bb[0], zero16);
 #pragma unroll
@@ -531,7 +537,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
             };
             if (HAS_C2P) {
 #pragma unroll
-                for (int rt = 0; rt < 3; ++rt) res[rt] = chain(fr[rt], qb);
+                for (int rt = 0; rt < (FIRST ? 3 : 2); ++rt) res[rt] = chain(fr[rt], qb);
             }
             if (HAS_P2C) {
                 res[3] = chain(fq[0], kb[0]);
@@ -560,6 +566,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
                 put_p(w, 1, res[4]);
                 put_p(4 + (w >> 1), w & 1, res[5]);
             }
+            if (HAS_C2P) res[2] = res[0];     // the carried tile of the next step
         };
 
         // First LDS stage of a tile: keys of steps 0 and 1 and the whole window of step 0 (192 rows of either
@@ -631,8 +638,8 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
             dl_next[0] = dl_step[0][0];
             dl_next[1] = dl_step[0][1];
             fetch();                      // window rows of step 1; they arrive under the products of step 0
-            load_frags(0, 0);
-            products();
+            load_frags(0, 0, std::true_type{});
+            products(std::true_type{});
             put_results();
             TDB_PSTAMP(2);
             phase_barrier();              // every position wave has its fragments of step 0
@@ -646,7 +653,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
             TDB_PSTAMP(4);
             phase_barrier();              // window of step 1 complete
             TDB_PSTAMP(5);
-            load_frags(off1, 1);
+            load_frags(off1, 1, std::false_type{});
             TDB_PSTAMP(6);
             // The tile after this one.  Its delta values are read at the end of the last step but one (when the fragment
             // and result registers are no longer needed); its first LDS stage is read from global memory and written
@@ -661,7 +668,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
                 constexpr bool TAIL = decltype(tail_tag)::value;   // step nsteps-2: no step s+2 to prepare
                 phase_barrier();          // scratch of step s complete
                 TDB_STAMP(0);
-                products();               // of step s+1, into registers; issued first: the wait for the
+                products(std::false_type{});   // of step s+1, into registers; issued first: the wait for the
                 __builtin_amdgcn_sched_barrier(0);  // prefetched global data then passes under the MFMAs
                 if (!TAIL) {
                     store(off2);          // new window rows of step s+2
@@ -673,7 +680,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
                 TDB_STAMP(2);
                 put_results();            // of step s+1
                 if (!TAIL) {
-                    load_frags(off2, s & 1);  // of step s+2
+                    load_frags(off2, s & 1, std::false_type{});  // of step s+2
                 } else {
                     read_deltas(nxt);
                 }
