@@ -503,21 +503,25 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         f32x16 res[6];
         auto load_frags = [&](int o, int kbuf, auto first_tag) {
             constexpr int C_TILES = decltype(first_tag)::value ? 3 : 2;   // (the third tile is carried, see products)
-            auto ring = [&](int x) { const int t = x + o; return t >= WIN ? t - WIN : t; };
+            // Window tiles are 32 rows and the ring offset is a multiple of 32, so a tile never straddles the wrap: the
+            // ring slot of a tile is scalar arithmetic, the lane only adds its row inside the tile.
+            auto ring_tile = [&](int t) { const int u = t + (o >> 5); return 32 * (u >= WIN / 32 ? u - WIN / 32 : u); };
+            const int lane_col = il * RS + 8 * hh;
             if (HAS_C2P) {
 #pragma unroll
                 for (int rt = 0; rt < C_TILES; ++rt) {
-                    const int row = ring(32 * w + 32 * rt + il);
+                    const uint16_t* base = sm.kr + ring_tile(w + rt) * RS;
 #pragma unroll
-                    for (int c = 0; c < 4; ++c) fr[rt][c] = lds_frag<X8>(sm.kr, row, 16 * c + 8 * hh);
+                    for (int c = 0; c < 4; ++c) fr[rt][c] = *reinterpret_cast<const X8*>(base + lane_col + 16 * c);
                 }
             }
             if (HAS_P2C) {
-                const int row3 = ring(32 * w + il), row4 = ring(32 * (4 + (w >> 1)) + il);
+                const uint16_t* base3 = sm.qr + ring_tile(w) * RS;
+                const uint16_t* base4 = sm.qr + ring_tile(4 + (w >> 1)) * RS;
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
-                    fq[0][c] = lds_frag<X8>(sm.qr, row3, 16 * c + 8 * hh);
-                    fq[1][c] = lds_frag<X8>(sm.qr, row4, 16 * c + 8 * hh);
+                    fq[0][c] = *reinterpret_cast<const X8*>(base3 + lane_col + 16 * c);
+                    fq[1][c] = *reinterpret_cast<const X8*>(base4 + lane_col + 16 * c);
                     kb[0][c] = lds_frag<X8>(sm.k[kbuf], il, 16 * c + 8 * hh);
                     kb[1][c] = lds_frag<X8>(sm.k[kbuf], 32 + il, 16 * c + 8 * hh);
                 }
