@@ -999,7 +999,23 @@ bool tdb_mfma_supported(const TdbKernelParams& p, int dtype) {
     return true;
 }
 
-hipError_t tdb_launch_mfma(const TdbKernelParams& p, int dtype, hipStream_t stream) {
+hipError_t tdb_launch_mfma(const TdbKernelParams& whole, int dtype, hipStream_t stream) {
+    // Packed batches of more than 64 sequences go out as several launches of at most 64 (even parts): the kernel
+    // balances a persistent launch from sequence boundaries held one per lane, which is worth ~20 % over handing
+    // every tile to a workgroup of its own.  A part is the same call with fewer sequences: cu_seqlens holds
+    // absolute token offsets, so only its start and the count move.
+    if (whole.varlen && whole.B > 64) {
+        const int parts = (whole.B + 63) / 64, per = (whole.B + parts - 1) / parts;
+        for (int first = 0; first < whole.B; first += per) {
+            TdbKernelParams part = whole;
+            part.cu_seqlens = whole.cu_seqlens + first;
+            part.B = whole.B - first < per ? whole.B - first : per;
+            const hipError_t e = tdb_launch_mfma(part, dtype, stream);
+            if (e != hipSuccess) return e;
+        }
+        return hipSuccess;
+    }
+    const TdbKernelParams& p = whole;
     const int64_t tiles = int64_t(p.varlen ? p.total / BM + p.B : p.B * ((p.L + BM - 1) / BM)) * p.H;
     const int64_t round = 8 * XCD_GROUP;                 // the id regrouping is a bijection on multiples of this
     const int nblocks = int((tiles + round - 1) / round * round);
@@ -1013,10 +1029,9 @@ hipError_t tdb_launch_mfma(const TdbKernelParams& p, int dtype, hipStream_t stre
         cus_of[dev] = n / 8 * 8;
     }
     // Persistent workgroups, one per CU: fixed layout with a strided deal (tiles cost about the same), packed
-    // batches of up to 64 sequences with a cost-balanced deal computed in the kernel.  Larger packed batches: every
-    // tile gets its own workgroup and the hardware dispatcher hands them to CUs as they free up.
+    // batches with a cost-balanced deal computed in the kernel.
     const int persistent = nblocks < cus_of[dev] ? nblocks : cus_of[dev];
-    const dim3 grid(unsigned(p.varlen && p.B > 64 ? nblocks : persistent)), block(NTHREADS);
+    const dim3 grid{unsigned(persistent)}, block(NTHREADS);
     const size_t smem = sizeof(Smem);
     const bool c2p = p.pk != nullptr, p2c = p.pq != nullptr;
 #define TDB_LAUNCH(A, B, T)                                                                                     \
