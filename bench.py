@@ -37,7 +37,7 @@ METRIC = "attn TFLOP/s + tokens/s, DeBERTa-v3-base b32xL512 bf16, fixed and varl
 # HBM bytes per launch from `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` runs of this script, each counter scaled
 # by what it reads for a plain 512 MiB device copy (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000); the runs and raw counter
 # values are recorded in profiles/attn_mfma_kernel_fixed_b32xL512.md and profiles/attn_mfma_kernel_varlen_64seq.md.
-MEASURED_TRAFFIC_BYTES = {"fixed": 106.7e6, "varlen": 213.5e6}
+MEASURED_TRAFFIC_BYTES = {"fixed": 104.1e6, "varlen": 210.3e6}
 
 
 def flops_of(lengths) -> float:
