@@ -8,8 +8,9 @@
 //     max / row sum are in-lane reductions plus one exchange between the half-waves, and the S^T
 //     accumulator registers are already the B operand of the P.V product, so probabilities never
 //     touch LDS.
-//   * 4 "position" waves: they stage K, V and the relative-position rows from global memory into
-//     LDS and compute, one key step ahead, the position products on the matrix cores.
+//   * 4 "position" waves: they stage the relative-position rows from global memory into LDS and
+//     compute, one key step ahead, the position products on the matrix cores.  (K and V are staged
+//     by the score waves.)
 //
 // Position terms, per key step (keys j0 .. j0+63), in "position space": the workgroup needs
 // relative positions r = i - j in a window of 128+64-1 values.  Rows K_r[delta(r)] and Q_r[delta(r)]
@@ -252,7 +253,9 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         }
         return false;
     };
-    // Packed launches of up to 64 sequences use a cost-balanced walk instead of the strided one: tiles differ in
+    // Packed launches of up to 64 sequences (the launcher splits larger batches, so that is every packed launch it
+    // makes; a larger one would take the strided walk with the tile numbering of `locate`) use a cost-balanced walk
+    // instead of the strided one: tiles differ in
     // length by up to 8x, so workgroup g takes a CONTIGUOUS range of the tile list (heads outermost, then sequences,
     // then the query tiles of a sequence) whose summed cost is 1/gridDim.x of the total.  The cost of a tile is
     // 8 * (its key steps) + 13, in eighths of a key step (13: what opening a tile costs).  Every wave derives the
@@ -373,16 +376,19 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     // window slides down by 64, so only its 64 lowest positions are fetched and they overwrite the 64 highest
     // of the previous step.  Window row x of step s sits in ring slot (x + off_s) mod 192, off_s = (128*s) mod 192.
     //
-    // A tile opens with three barriers (first stage in LDS; position products of step 0 in the scratch; window of
-    // step 1 complete).  Then each step has two halves separated by workgroup barriers, arranged so that in either
-    // half one role is on the LDS and the other on the matrix cores:
-    //   A  score waves read this step's position terms out of the C'/P' scratch into their score accumulators;
-    //      position waves hand register-prefetched global data to LDS (keys of step s+2, values of step s, 64 window
-    //      rows of step s+2) and run the 24 position MFMAs of step s+1 on fragments they already hold;
-    //   B  score waves: S^T(s), softmax(s), P.V(s), and they pick up the K fragments of step s+1;
-    //      position waves: results of step s+1 into the now free scratch, global fetches for the next half A,
-    //      LDS fragments of step s+2.
-    // Both roles pass 3 + 2*nsteps barriers per tile and walk the same tile list.
+    // A tile opens with its first stage in LDS (written during the last step of the tile before; for the first tile of
+    // the workgroup by all threads) and two barriers: position products of step 0 in the scratch; window of step 1
+    // complete.  Then each step has two halves separated by workgroup barriers, arranged so that in either half one
+    // role leans on the LDS and the other on the matrix cores:
+    //   A  score waves read this step's position terms out of the C'/P' scratch into their score accumulators and
+    //      hand register-prefetched keys (step s+2) and values (step s) to LDS; position waves run the 20 position
+    //      MFMAs of step s+1 on fragments they already hold, then store the 64 new window rows of step s+2 and
+    //      request those of step s+3;
+    //   B  score waves: S^T(s), softmax(s), P.V(s); they pick up the K fragments of step s+1 and request keys and
+    //      values for the next half A; position waves: results of step s+1 into the now free scratch, LDS fragments
+    //      of step s+2.
+    // Both roles pass 2 + 2*nsteps barriers per tile (the barrier that ends the last step is also the one after which
+    // the next tile's first stage is visible) and walk the same tile list.
     const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     auto prev_off = [](int o) { return o >= BN ? o - BN : o + WIN - BN; };   // ring offset of the following step
 
