@@ -188,6 +188,12 @@ def test_eval_caches_follow_weight_updates():
     fresh = model(input_ids=ids, attention_mask=mask).last_hidden_state.detach()
     assert (changed[valid] - fresh[valid]).abs().max() <= 1e-5 * fresh[valid].abs().max()
     assert (changed[valid] - first[valid]).abs().max() > 1e-3
+    with torch.no_grad():                                                                # relative embeddings updated in place
+        model.encoder.rel_embeddings.weight[:, :16].mul_(-3.0)                           # (not a rescaling: the LayerNorm would undo one)
+        moved = model(input_ids=ids, attention_mask=mask).last_hidden_state
+    fresh2 = model(input_ids=ids, attention_mask=mask).last_hidden_state.detach()
+    assert (moved[valid] - fresh2[valid]).abs().max().item() <= 1e-5 * fresh2[valid].abs().max().item()
+    assert (moved[valid] - changed[valid]).abs().max().item() > 1e-4
     with torch.no_grad():                                                                # shorter sequences, new mask
         mask2 = mask.clone()
         mask2[:, -3:] = 0

@@ -54,8 +54,9 @@ from .padding import _get_unpad_data, index_first_axis, key_padding_mask, pad_in
 
 
 def _versions(*tensors):
-    """Identity of a set of tensors for cache keys: storage address and in-place modification counter."""
-    return tuple((t.data_ptr(), t._version, t.dtype, t.device) if t is not None else None for t in tensors)
+    """Identity of a set of live tensors (parameters) for cache keys: object, storage address and in-place
+    modification counter.  Only meaningful for tensors that stay alive between the calls that compare keys."""
+    return tuple((id(t), t.data_ptr(), t._version, t.dtype, t.device) if t is not None else None for t in tensors)
 
 
 def _lengths_of(attention_mask):
@@ -162,7 +163,15 @@ class FlashDisentangledSelfAttention(DisentangledSelfAttention):
         projection weights have been modified (or moved / cast)."""
         kp = self.key_proj if self.share_att_key else getattr(self, "pos_key_proj", None)
         qp = self.query_proj if self.share_att_key else getattr(self, "pos_query_proj", None)
-        key = (_versions(rel_embeddings, *(t for m in (kp, qp) if m is not None for t in (m.weight, m.bias))), dtype)
+        # Identity of the relative embeddings: the encoder's layer-normed copy is a temporary, whose address says
+        # nothing (it can be reused by a later, different tensor); FlashDebertaV2Encoder tags what it hands out with
+        # the identity of its sources.  A parameter speaks for itself.  Anything else is not cached.
+        source = getattr(rel_embeddings, "_tdb_source", None)
+        if source is None and isinstance(rel_embeddings, nn.Parameter):
+            source = _versions(rel_embeddings)
+        if source is None:
+            return self._project_tables(rel_embeddings[0:2 * self.pos_ebd_size])
+        key = (source, _versions(*(t for m in (kp, qp) if m is not None for t in (m.weight, m.bias))), dtype)
         cached = self.__dict__.get("_tdb_tables")
         if cached is None or cached[0] != key:
             rel = rel_embeddings[0:2 * self.pos_ebd_size]                # dropout is the identity in eval mode
@@ -216,6 +225,26 @@ class FlashDebertaV2Encoder(DebertaV2Encoder):
     def __init__(self, config):
         super().__init__(config)
         self.layer = nn.ModuleList([FlashDebertaV2Layer(config) for _ in range(config.num_hidden_layers)])
+
+    def get_rel_embedding(self):
+        """As the parent (modeling_deberta_v2.py:593-597); in eval mode under ``no_grad`` the (layer-normed) result is
+        computed once per state of its sources and tagged with their identity, which the attention modules key
+        their position-table caches on."""
+        if self.training or torch.is_grad_enabled() or not self.relative_attention:
+            return super().get_rel_embedding()
+        sources = [self.rel_embeddings.weight]
+        if "layer_norm" in self.norm_rel_ebd:
+            sources += [self.LayerNorm.weight, self.LayerNorm.bias]
+        key = _versions(*sources)
+        cached = self.__dict__.get("_tdb_rel")
+        if cached is None or cached[0] != key:
+            rel = super().get_rel_embedding()
+            if rel is self.rel_embeddings.weight:
+                rel = rel.detach()           # a tensor of its own to carry the tag (shares the storage)
+            rel._tdb_source = key
+            cached = (key, rel)
+            self.__dict__["_tdb_rel"] = cached
+        return cached[1]
 
     def forward(self, hidden_states, attention_mask, output_hidden_states=True, output_attentions=False,
                 query_states=None, relative_pos=None, return_dict=True):
