@@ -233,8 +233,9 @@ def test_bf16_varlen_vs_oracle(force_generic):
 
 @pytest.mark.parametrize("force_generic", [False, True])
 def test_bf16_varlen_more_than_64_sequences(force_generic):
-    """150 short sequences: the wave-wide scan over the packed boundaries needs three chunks of 64, of which only
-    the first is kept in registers by the matrix-core kernel."""
+    """150 short sequences, more than the 64 whose boundaries a wave holds in its lanes: the matrix-core path goes out
+    as three launches of 50 (the result must equal, bit for bit, what separate calls on the three parts give), the
+    vector-ALU kernel scans the boundaries in chunks of 64."""
     H, D, buckets, max_rel = 2, 64, 256, 512
     rs = np.random.RandomState(4)
     lengths = [int(x) for x in rs.randint(1, 200, size=150)]
@@ -250,6 +251,15 @@ def test_bf16_varlen_more_than_64_sequences(force_generic):
         max(lengths), max(lengths), False, 1 / math.sqrt(3 * D), buckets, max_rel,
         pos_key_layer=inp["pk"].to(DEV), pos_query_layer=inp["pq"].to(DEV), force_generic=force_generic)
     assert_close_bf16(out.cpu(), ref, "bf16 varlen, 150 sequences", tol=1e-2)
+    if not force_generic:
+        for first in (0, 50, 100):
+            lo, hi = int(cu[first]), int(cu[first + 50])
+            part_cu = (cu[first:first + 51] - cu[first]).to(DEV)
+            part = flash_attention_with_disentangled_varlen(
+                packed["q"][lo:hi].to(DEV), packed["k"][lo:hi].to(DEV), packed["v"][lo:hi].to(DEV), None, None, part_cu,
+                part_cu, max(lengths), max(lengths), False, 1 / math.sqrt(3 * D), buckets, max_rel,
+                pos_key_layer=inp["pk"].to(DEV), pos_query_layer=inp["pq"].to(DEV))
+            assert torch.equal(part, out[lo:hi]), f"sequences {first}..{first + 49}"
 
 
 @pytest.mark.parametrize("force_generic", [False, True])
