@@ -150,7 +150,7 @@ def cpu_baseline(tensors, lengths, budget_s=12.0):
                       f"float32 torch-CPU oracle, median of {len(times)} runs"}
 
 
-def model_benchmark(dev, steps=10, warmup=3):
+def model_benchmark(dev, steps=30, warmup=10):
     """End-to-end forward of a DeBERTa-v3-large-shaped model (24 layers x 1024, 16 heads x 64, FFN 4096, vocabulary
     128100, buckets 256, max_rel 512, shared keys, c2p|p2c, layer-normed relative embeddings; random N(0, 0.02)
     weights, eval mode, bf16) on ids [16, 512] with right-padded lengths U[64, 512]: valid tokens per second with the
