@@ -7,21 +7,33 @@
 //     softmax, O^T += V^T.P^T.  Scores are kept transposed so that a lane owns ONE query row: row
 //     max / row sum are in-lane reductions plus one exchange between the half-waves, and the S^T
 //     accumulator registers are already the B operand of the P.V product, so probabilities never
-//     touch LDS.
+//     touch LDS.  Wave w owns the query rows  row0 + 4n + w  (n = lane & 31): rows are dealt to the
+//     waves round robin, which is what makes the c2p ring below addressable with aligned vectors.
 //   * 4 "position" waves: they stage the relative-position rows from global memory into LDS and
 //     compute, one key step ahead, the position products on the matrix cores.  (K and V are staged
 //     by the score waves.)
 //
-// Position terms, per key step (keys j0 .. j0+63), in "position space": the workgroup needs
-// relative positions r = i - j in a window of 128+64-1 values.  Rows K_r[delta(r)] and Q_r[delta(r)]
-// of the per-head tables are staged in LDS for that window (delta from the host-built table, so log
-// bucketing, saturation beyond max_relative_positions and the un-bucketed case are one code path
-// with bit-exact indices).  Then
-//   c2p:  C'^T[r, i] = K_r'[r] . Q_i      per 32-query block, over its own 96-position sub-window,
-//   p2c:  P'^T[r, j] = Q_r'[r] . K_j      once per workgroup,
-// both on MFMA, written to LDS (c2p as fp32, p2c as bf16) and read back skewed by the score waves:
-// score (i, j) takes C'[i][i-j] and P'[j][i-j], i.e. Q_i.K_r[delta(i-j)] + K_j.Q_r[delta(i-j)], the
-// Hugging Face eager definition (modeling_deberta_v2.py:317-324, :337-343).
+// Position terms, in "position space" (relative position r = i - j; delta(r) comes from the
+// host-built table, so log bucketing, saturation beyond max_relative_positions and the un-bucketed
+// case are one code path with bit-exact indices).  Key step s covers keys 64s .. 64s+63 and touches
+// the window r = B_s .. B_s + 190, B_s = row0 - 64s - 63; rows K_r[delta(r)] and Q_r[delta(r)] of the
+// per-head tables for that window live in two 192-row LDS rings (each step fetches the 64 new rows).
+//   c2p:  every relative position a query meets is met exactly once, so the products
+//         C'[i][r] = Q_i . K_r[delta(r)] are computed once per (query, position): each step the
+//         position wave of query block w contracts only the 64 positions that are new to the block
+//         (2 MFMA tiles) and files the results, as bf16, under the KEY they belong to (j = i - r) in
+//         a per-query ring of 192 key slots.  Because the rows of a wave are 4 apart, four consecutive
+//         positions of the MFMA result land on four consecutive keys at a 4-aligned slot for every
+//         lane: 8-byte stores going in, and the score wave reads the 8 consecutive keys an MFMA B
+//         operand holds with one 16-byte load and adds them to the score accumulators with an MFMA
+//         against an identity fragment -- no per-element gather, no unpacking.
+//   p2c:  P'^T[r, j] = Q_r[delta(r)] . K_j for the window of the step (10 MFMA tiles: the corners
+//         of the window that no (query, key) pair of the tile reaches are skipped), written to LDS
+//         as bf16 P'[j][r - B_s] and read back skewed by the score waves: score (i, j) takes
+//         P'[j][i - j - B_s], which becomes the initial value of the S^T accumulator.
+// Together: S[i,j] = Q_i.K_j + Q_i.K_r[delta(i-j)] + K_j.Q_r[delta(i-j)], the Hugging Face eager
+// definition (modeling_deberta_v2.py:317-324, :337-343).
+#include <mutex>
 #include <type_traits>
 #include <utility>
 
@@ -46,9 +58,10 @@ constexpr int BN = 64;              // keys per step
 constexpr int D = 64;
 constexpr int NTHREADS = 512;       // 4 score waves + 4 position waves
 constexpr int WIN = BM + BN;        // ring of staged window rows (one more than the 191 positions in use)
-constexpr int RS = 72;              // LDS row stride (elements) of 64-wide bf16 rows: 144 B, conflict-free b128
-constexpr int CS = 100;             // row stride (floats) of the per-block c2p scratch [32][96 used]
-constexpr int PS = 196;             // row stride of the p2c scratch                   [64][192 used]
+constexpr int RS = 72;              // LDS row stride (elements) of 64-wide 16-bit rows: 144 B, conflict-free b128
+constexpr int CRING = 192;          // key slots of the c2p ring of one query row
+constexpr int CRS = 200;            // its row stride (elements): 400 B, so that 32 rows read 16 B or write 8 B on distinct banks
+constexpr int PS = 196;             // row stride (elements) of the p2c scratch [64 keys][191 positions]
 constexpr int RSRC_FLAGS = 0x00020000;   // raw buffer resource, 32-bit data format
 constexpr int XCD_GROUP = 4;        // query tiles of one (sequence, head) kept on one XCD
 
@@ -57,14 +70,14 @@ struct Smem {
     uint16_t v[BN * RS];
     uint16_t kr[WIN * RS];
     uint16_t qr[WIN * RS];
-    float c[4][32 * CS];
+    uint16_t c[BM * CRS];               // c2p ring: row 32w + n belongs to query row0 + 4n + w, slot = key mod 192
     uint16_t p[BN * PS];
 };
 
 // The two 16-bit element types the kernel is instantiated for: what differs is the MFMA and the float conversion.
 // (No dot-product instructions anywhere: v_dot2 runs on the matrix pipe and would queue behind the other role's MFMAs,
 // while plain vector instructions run beside them.)  (bf16: fp32's range, 8 significant bits; fp16: 11 bits, range 65504 --
-// the p2c products are stored in the element type, the probabilities are at most 2^8.)
+// the position products are stored in the element type, the probabilities are at most 2^8.)
 template <int DT>
 struct Elem;
 template <>
@@ -73,11 +86,7 @@ struct Elem<TDB_BF16> {
     using X2 = bf16x2;
     using X8 = bf16x8;
     static __device__ __forceinline__ f32x16 mfma(X8 a, X8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
-    // One half of a dword as fp32 through a byte permute (the selector says which half): bf16 -> fp32 is a shift.
-    static constexpr uint32_t PICK_LO = 0x05040c0cu, PICK_HI = 0x07060c0cu;
-    static __device__ __forceinline__ float pick(uint32_t pair, uint32_t sel) {
-        return __builtin_bit_cast(float, __builtin_amdgcn_perm(pair, 0u, sel));
-    }
+    static __device__ __forceinline__ float widen(uint16_t raw) { return __builtin_bit_cast(float, uint32_t(raw) << 16); }
 };
 template <>
 struct Elem<TDB_F16> {
@@ -85,10 +94,7 @@ struct Elem<TDB_F16> {
     using X2 = f16x2;
     using X8 = f16x8;
     static __device__ __forceinline__ f32x16 mfma(X8 a, X8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
-    static constexpr uint32_t PICK_LO = 0x0c0c0504u, PICK_HI = 0x0c0c0706u;
-    static __device__ __forceinline__ float pick(uint32_t pair, uint32_t sel) {
-        return (float)__builtin_bit_cast(X2, __builtin_amdgcn_perm(pair, 0u, sel))[0];
-    }
+    static __device__ __forceinline__ float widen(uint16_t raw) { return (float)__builtin_bit_cast(_Float16, raw); }
 };
 
 template <typename X8>
@@ -97,60 +103,13 @@ __device__ __forceinline__ X8 lds_frag(const uint16_t* row_base, int row, int co
 }
 
 template <typename E>
-__device__ __forceinline__ u32x2 pack4(float a, float b, float c, float d) {
-    typename E::X2 lo = {(typename E::T)a, (typename E::T)b};
-    typename E::X2 hi = {(typename E::T)c, (typename E::T)d};
-    u32x2 r;
-    r[0] = __builtin_bit_cast(uint32_t, lo);
-    r[1] = __builtin_bit_cast(uint32_t, hi);
-    return r;
+__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+    typename E::X2 v = {(typename E::T)lo, (typename E::T)hi};
+    return __builtin_bit_cast(uint32_t, v);
 }
 
 // Workgroup barrier that instruction scheduling may not move anything across either: register-only work (MFMAs,
 // address arithmetic) stays in the pipeline half it was written in.
-#ifdef TDB_TIMING
-// Development aid (off in the library build): cycle stamps of one workgroup's first score wave and first position
-// wave, summed per pipeline phase, and entry / exit wall-clock times of every workgroup.
-__device__ long long tdb_timing[16];
-__device__ long long tdb_ptiming[16];
-__device__ long long tdb_wtiming[8 * 6];    // the six phase sums of every wave of that workgroup
-__device__ long long tdb_trace[4 * 4096];   // per workgroup: entry, exit (100 MHz wall clock), hardware id, steps
-#define TDB_T_ENTRY const long long t_entry = __builtin_readcyclecounter(); const long long t_wall = wall_clock64(); \
-        long long t_pro[8] = {0, 0, 0, 0, 0, 0, 0, 0}; long long t_plast = t_entry;
-#define TDB_PSTAMP(slot) do { __builtin_amdgcn_sched_barrier(0); const long long t_now = __builtin_readcyclecounter(); \
-        t_pro[slot] += t_now - t_plast; t_plast = t_now; __builtin_amdgcn_sched_barrier(0); } while (0)
-#define TDB_PRESET do { t_plast = __builtin_readcyclecounter(); } while (0)
-#define TDB_P_FLUSH do { if (blockIdx.x == TDB_TIMING && (threadIdx.x & 255) == 0) \
-        for (int t_i = 0; t_i < 8; ++t_i) tdb_ptiming[t_i + (threadIdx.x >> 8) * 8] = t_pro[t_i]; } while (0)
-#define TDB_T_DECL long long t_acc[6] = {0, 0, 0, 0, 0, 0}; long long t_last = __builtin_readcyclecounter(); t_acc[4] = t_last - t_entry;
-// (A stamp is a scalar memory read: it drains the wave's LDS queue and costs about 150 cycles.  TDB_TIMING_LIGHT keeps
-// only the stamps right after a barrier: slot 0 = half B + barrier, slot 2 = half A + barrier.)
-#ifdef TDB_TIMING_LIGHT
-#define TDB_STAMP(slot) do { if ((slot) == 0 || (slot) == 2) { __builtin_amdgcn_sched_barrier(0); const long long t_now = __builtin_readcyclecounter(); \
-        t_acc[slot] += t_now - t_last; t_last = t_now; __builtin_amdgcn_sched_barrier(0); } } while (0)
-#else
-#define TDB_STAMP(slot) do { __builtin_amdgcn_sched_barrier(0); const long long t_now = __builtin_readcyclecounter(); \
-        t_acc[slot] += t_now - t_last; t_last = t_now; __builtin_amdgcn_sched_barrier(0); } while (0)
-#endif
-#define TDB_T_FLUSH(base) do { if (blockIdx.x == TDB_TIMING && (threadIdx.x & 255) == 0) \
-        for (int t_i = 0; t_i < 6; ++t_i) tdb_timing[(base) + t_i] = t_acc[t_i]; \
-        if (blockIdx.x == TDB_TIMING && (threadIdx.x & 63) == 0) \
-        for (int t_i = 0; t_i < 6; ++t_i) tdb_wtiming[(threadIdx.x >> 6) * 6 + t_i] = t_acc[t_i]; } while (0)
-#define TDB_TRACE_EXIT do { if (threadIdx.x == 0 && blockIdx.x < 4096) { \
-        tdb_trace[4 * blockIdx.x] = t_wall; tdb_trace[4 * blockIdx.x + 1] = wall_clock64(); \
-        tdb_trace[4 * blockIdx.x + 2] = (long long)__builtin_amdgcn_s_getreg(63492) | ((long long)__builtin_amdgcn_s_getreg((31 << 11) | 20) << 32); \
-        tdb_trace[4 * blockIdx.x + 3] = nsteps; } } while (0)
-#else
-#define TDB_T_ENTRY
-#define TDB_PSTAMP(slot)
-#define TDB_PRESET
-#define TDB_P_FLUSH
-#define TDB_T_DECL
-#define TDB_STAMP(slot)
-#define TDB_T_FLUSH(base)
-#define TDB_TRACE_EXIT
-#endif
-
 __device__ __forceinline__ void phase_barrier() {
     __builtin_amdgcn_sched_barrier(0);
     __syncthreads();
@@ -167,7 +126,6 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     Smem& sm = *reinterpret_cast<Smem*>(smem_raw);
     constexpr bool HAS_POS = HAS_C2P || HAS_P2C;
 
-    TDB_T_ENTRY
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const bool score_role = wave < 4;     // waves 0..3 score, 4..7 position; wave w and w+4 share query block w
@@ -189,7 +147,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     struct Tile {
         int vb, head, b, row0, len;       // vb < 0: no tile
         int64_t tok0;
-        int cost;                         // balanced walk: cost coordinate of the tile (see below)
+        int64_t cost;                     // balanced walk: cost coordinate of the tile (see below)
     };
     auto tile_index = [&](int vb, int& hd, int& tile_id) {   // false: the virtual block has no tile
         const int xcd = vb & 7, slot = vb >> 3;
@@ -260,11 +218,18 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     // then the query tiles of a sequence) whose summed cost is 1/gridDim.x of the total.  The cost of a tile is
     // 8 * (its key steps) + 13, in eighths of a key step (13: what opening a tile costs).  Every wave derives the
     // same ranges from the boundaries in its lanes; a tile belongs to the workgroup whose cost interval holds the
-    // tile's start coordinate.  Consecutive query tiles of a sequence then run back to back on one CU.
-    const bool balanced = p.varlen && p.B <= 64;
-    int n_lane = 0, pre_lane = 0, cost_per_head = 0, cost_end = 0;
+    // tile's start coordinate.  Consecutive query tiles of a sequence then run back to back on one CU.  Cost
+    // coordinates are 64-bit: one sequence of 2^20 tokens alone costs 2^30.
+    bool balanced = p.varlen && p.B <= 64;
+    int n_lane = 0;
+    int64_t pre_lane = 0, cost_per_head = 0, cost_end = 0;
     auto tiles_of = [](int n) { return (n + BM - 1) / BM; };
-    auto cost_of = [](int n) { return 8 * ((n + BN - 1) / BN) + 13; };
+    auto cost_of = [](int n) { return int64_t(8 * ((n + BN - 1) / BN) + 13); };
+    auto lane64 = [](int64_t v, int lane) {
+        const int lo = __builtin_amdgcn_readlane(int(uint32_t(uint64_t(v))), lane);
+        const int hi = __builtin_amdgcn_readlane(int(uint32_t(uint64_t(v) >> 32)), lane);
+        return int64_t((uint64_t(uint32_t(hi)) << 32) | uint32_t(lo));
+    };
     if (balanced) {
         if (l < p.B) {
             n_lane = cu_hi - cu_lo;
@@ -274,10 +239,10 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         pre_lane = tiles_of(n_lane) * cost_of(n_lane);                    // inclusive prefix sum over the wave
 #pragma unroll
         for (int d = 1; d < 64; d <<= 1) {
-            const int up = __shfl_up(pre_lane, d);
+            const int64_t up = __shfl_up(pre_lane, d);
             if (l >= d) pre_lane += up;
         }
-        cost_per_head = __builtin_amdgcn_readlane(pre_lane, 63);
+        cost_per_head = lane64(pre_lane, 63);
     }
     // Moves (head, sequence, tile) forward until it names an existing tile; t.cost is its start coordinate.
     auto settle = [&](Tile t, int tile_in_seq) {
@@ -307,19 +272,20 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     auto first_balanced = [&]() {
         Tile t;
         t.vb = -1;
-        t.head = t.b = t.row0 = t.len = t.cost = 0;
+        t.head = t.b = t.row0 = t.len = 0;
+        t.cost = 0;
         t.tok0 = 0;
         if (cost_per_head <= 0) return t;
-        const int64_t total = int64_t(cost_per_head) * p.H;
-        const int start = int(total * blockIdx.x / gridDim.x);
-        cost_end = int(total * (blockIdx.x + 1) / gridDim.x);
-        t.head = start / cost_per_head;
-        const int rem = start - t.head * cost_per_head;
+        const int64_t total = cost_per_head * p.H;           // < 2^30 * 64 * 2^16: no overflow; the products below
+        const int64_t start = total / gridDim.x * blockIdx.x + total % gridDim.x * blockIdx.x / gridDim.x;   // stay below 2^63 too
+        cost_end = total / gridDim.x * (blockIdx.x + 1) + total % gridDim.x * (blockIdx.x + 1) / gridDim.x;
+        t.head = int(start / cost_per_head);
+        const int64_t rem = start - t.head * cost_per_head;
         const unsigned long long owners = __builtin_amdgcn_ballot_w64(pre_lane > rem);
         t.b = __builtin_amdgcn_readfirstlane(__builtin_ctzll(owners));
         const int n = __builtin_amdgcn_readlane(n_lane, t.b);
-        const int before = __builtin_amdgcn_readlane(pre_lane, t.b) - tiles_of(n) * cost_of(n);
-        const int tile_in_seq = (rem - before + cost_of(n) - 1) / cost_of(n);     // first tile starting at or after rem
+        const int64_t before = lane64(pre_lane, t.b) - tiles_of(n) * cost_of(n);
+        const int tile_in_seq = int((rem - before + cost_of(n) - 1) / cost_of(n));     // first tile starting at or after rem
         t.cost = t.head * cost_per_head + before + tile_in_seq * cost_of(n);
         return settle(t, tile_in_seq);
     };
@@ -334,7 +300,8 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     auto find_tile = [&](int vb) {
         Tile t;
         t.vb = -1;
-        t.head = t.b = t.row0 = t.len = t.cost = 0;
+        t.head = t.b = t.row0 = t.len = 0;
+        t.cost = 0;
         t.tok0 = 0;
         for (; vb < nblocks; vb += gridDim.x) {
             int hd, tile_id;
@@ -375,20 +342,29 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     // The rows K_r[delta(r)] / Q_r[delta(r)] of that window live in a 192-row ring: going to the next step the
     // window slides down by 64, so only its 64 lowest positions are fetched and they overwrite the 64 highest
     // of the previous step.  Window row x of step s sits in ring slot (x + off_s) mod 192, off_s = (128*s) mod 192.
+    // The 64 + 3 lowest rows of the window are exactly the positions that are new to the four query blocks
+    // (block w: window rows w .. w+63), i.e. what the c2p products of the step contract.
     //
     // A tile opens with its first stage in LDS (written during the last step of the tile before; for the first tile of
-    // the workgroup by all threads) and two barriers: position products of step 0 in the scratch; window of step 1
+    // the workgroup by all threads) and two barriers: position products of step 0 in LDS; window of step 1
     // complete.  Then each step has two halves separated by workgroup barriers, arranged so that in either half one
     // role leans on the LDS and the other on the matrix cores:
-    //   A  score waves read this step's position terms out of the C'/P' scratch into their score accumulators and
-    //      hand register-prefetched keys (step s+2) and values (step s) to LDS; position waves run the 20 position
-    //      MFMAs of step s+1 on fragments they already hold, then store the 64 new window rows of step s+2 and
-    //      request those of step s+3;
-    //   B  score waves: S^T(s), softmax(s), P.V(s); they pick up the K fragments of step s+1 and request keys and
-    //      values for the next half A; position waves: results of step s+1 into the now free scratch, LDS fragments
-    //      of step s+2.
+    //   A  score waves read this step's position terms (c2p ring fragments, P' scratch), hand register-prefetched
+    //      keys (step s+2) and values (step s) to LDS, run the S^T(s) MFMAs on top of the position terms and pick up
+    //      the K fragments of step s+1; position waves run the c2p MFMAs of step s+1 on fragments they already hold,
+    //      then store the 64 new window rows of step s+2 and request those of step s+3;
+    //   B  score waves: softmax(s), P.V(s), and they request keys and values for the next half A; position waves:
+    //      c2p results of step s+1 into the ring, the p2c MFMAs of step s+1 and their results into the now free
+    //      scratch, LDS fragments of step s+2.
+    // (Each half so carries half of the step's MFMAs and half of its LDS traffic.)
     // Both roles pass 2 + 2*nsteps barriers per tile (the barrier that ends the last step is also the one after which
     // the next tile's first stage is visible) and walk the same tile list.
+    //
+    // c2p ring bookkeeping.  "Batch" t is the set of positions new at step t: for block w, r = row0 + w - 64t - 63 + m,
+    // m = 0..63; lane n of the block (query row0 + 4n + w) meets them at keys 64t + 63 + 4n - m.  A tile opens with
+    // batches -2, -1, 0 (together the 188 positions step 0 needs; the part that falls on negative keys lands in slots
+    // that their proper batch rewrites before anybody reads them).  Batch t+1 is written in half B of step t, after the
+    // score waves have read the keys of step t; the slots it overwrites held keys below 64(t+1).
     const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     auto prev_off = [](int o) { return o >= BN ? o - BN : o + WIN - BN; };   // ring offset of the following step
 
@@ -415,7 +391,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     X8 qb[4];
     auto load_q = [&](X8 (&dst)[4], const Tile& t) {
         const uint16_t* Qt = static_cast<const uint16_t*>(p.q) + (p.varlen ? t.tok0 * p.qs_l : int64_t(t.b) * p.qs_b) + int64_t(t.head) * p.qs_h;
-        const int qrow = t.row0 + 32 * w + il;
+        const int qrow = t.row0 + 4 * il + w;
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             u32x4 x = {0, 0, 0, 0};
@@ -500,84 +476,108 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
             }
         };
         // Position products of one key step, in three stages that the pipeline places in different halves:
-        //   load_frags  MFMA operands out of LDS: K_r' rows of the 96-position sub-window of query block w (fr),
-        //               Q_r' rows of position tiles w and 4 + w/2 of the workgroup window (fq), both key tiles (kb);
-        //   products    c2p  C'^T[r, i] = K_r'[r].Q_i  (3 tiles),  p2c  P'^T[r, j] = Q_r'[r].K_j  (wave w: tile w
-        //               against both key tiles, and tile (4 + w/2, w & 1)) -- 24 MFMAs;
-        //   put_results c2p as fp32 C'[i][r'], p2c as bf16 P'[j][r''] into the scratch.
-        X8 fr[3][4], fq[2][4], kb[2][4];
-        f32x16 res[6];
-        auto load_frags = [&](int o, int kbuf, auto first_tag) {
-            constexpr int C_TILES = decltype(first_tag)::value ? 3 : 2;   // (the third tile is carried, see products)
+        //   load_frags   MFMA operands out of LDS: for c2p the K_r' rows of window rows xb + 32 rt + m (xb = w: the
+        //                64 positions new to query block w; the tiles are not aligned to the 32-row ring tiles, so each
+        //                lane wraps its own row); for p2c the Q_r' rows of window tile w + 1 and, for waves 0 and 1,
+        //                of tiles 0 and 5, and both key tiles (kb);
+        //   products     c2p  C'^T[r, i] = K_r'[r].Q_i  (2 tiles),  p2c  P'^T[r, j] = Q_r'[r].K_j  (wave w: tile w + 1
+        //                against both key tiles; wave 0: tile 0 against keys 32..63; wave 1: tile 5 against keys
+        //                0..31; the other two corners of the window are never read) -- results packed to 16 bits;
+        //   put_results  c2p into the ring (8-byte stores at 4-aligned key slots), p2c as P'[j][r''] into the scratch.
+        X8 fr[2][4], fq[2][4], kb[2][4];
+        u32x2 cpk[2][4], ppk[3][4];
+        const int lane_col = il * RS + 8 * hh;
+        auto load_fr = [&](int o, int xb) {
+            if (HAS_C2P) {
+#pragma unroll
+                for (int rt = 0; rt < 2; ++rt) {
+                    int slot = min(xb + 32 * rt + il, WIN - 1) + o;     // rows past the window: any row will do (negative keys)
+                    slot = slot >= WIN ? slot - WIN : slot;
+                    const uint16_t* base = sm.kr + slot * RS + 8 * hh;
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) fr[rt][c] = *reinterpret_cast<const X8*>(base + 16 * c);
+                }
+            }
+        };
+        auto load_fp = [&](int o, int kbuf) {
             // Window tiles are 32 rows and the ring offset is a multiple of 32, so a tile never straddles the wrap: the
             // ring slot of a tile is scalar arithmetic, the lane only adds its row inside the tile.
             auto ring_tile = [&](int t) { const int u = t + (o >> 5); return 32 * (u >= WIN / 32 ? u - WIN / 32 : u); };
-            const int lane_col = il * RS + 8 * hh;
-            if (HAS_C2P) {
-#pragma unroll
-                for (int rt = 0; rt < C_TILES; ++rt) {
-                    const uint16_t* base = sm.kr + ring_tile(w + rt) * RS;
-#pragma unroll
-                    for (int c = 0; c < 4; ++c) fr[rt][c] = *reinterpret_cast<const X8*>(base + lane_col + 16 * c);
-                }
-            }
             if (HAS_P2C) {
-                const uint16_t* base3 = sm.qr + ring_tile(w) * RS;
-                const uint16_t* base4 = sm.qr + ring_tile(4 + (w >> 1)) * RS;
+                const uint16_t* base3 = sm.qr + ring_tile(w + 1) * RS;
+                const uint16_t* base4 = sm.qr + ring_tile(w == 1 ? 5 : 0) * RS;
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
                     fq[0][c] = *reinterpret_cast<const X8*>(base3 + lane_col + 16 * c);
-                    fq[1][c] = *reinterpret_cast<const X8*>(base4 + lane_col + 16 * c);
+                    if (w < 2) fq[1][c] = *reinterpret_cast<const X8*>(base4 + lane_col + 16 * c);
                     kb[0][c] = lds_frag<X8>(sm.k[kbuf], il, 16 * c + 8 * hh);
                     kb[1][c] = lds_frag<X8>(sm.k[kbuf], 32 + il, 16 * c + 8 * hh);
                 }
             }
         };
-        // c2p: from one key step to the next the sub-window moves down by 64 positions, so its third tile (positions
-        // 64..95) is the first tile of the step before -- same K_r' rows, same queries, same products.  Only step 0
-        // computes three tiles; later steps compute two and write the carried one (copied to res[2] after it was
-        // written as the first tile) again at its new place.
-        auto products = [&](auto first_tag) {
-            constexpr bool FIRST = decltype(first_tag)::value;
-            auto chain = [&](const X8 (&a)[4], const X8 (&bb)[4]) {
-                f32x16 acc = E::mfma(a[0], bb[0], zero16);
+        auto chain = [&](const X8 (&a)[4], const X8 (&bb)[4]) {
+            f32x16 acc = E::mfma(a[0], bb[0], zero16);
 #pragma unroll
-                for (int c = 1; c < 4; ++c) acc = E::mfma(a[c], bb[c], acc);
-                return acc;
-            };
+            for (int c = 1; c < 4; ++c) acc = E::mfma(a[c], bb[c], acc);
+            return acc;
+        };
+        // c2p results, key order: register 4a + t of a tile holds position row 8a + 4hh + t, i.e. key k0 - t; the four
+        // keys k0-3 .. k0 of a group go out together, lowest key first.
+        auto pack_c = [&](const f32x16& acc, u32x2 (&out)[4]) {
+#pragma unroll
+            for (int a = 0; a < 4; ++a)
+                out[a] = u32x2{pack2<E>(acc[4 * a + 3], acc[4 * a + 2]), pack2<E>(acc[4 * a + 1], acc[4 * a])};
+        };
+        auto pack_p = [&](const f32x16& acc, u32x2 (&out)[4]) {
+#pragma unroll
+            for (int a = 0; a < 4; ++a)
+                out[a] = u32x2{pack2<E>(acc[4 * a], acc[4 * a + 1]), pack2<E>(acc[4 * a + 2], acc[4 * a + 3])};
+        };
+        auto products_c = [&]() {
             if (HAS_C2P) {
 #pragma unroll
-                for (int rt = 0; rt < (FIRST ? 3 : 2); ++rt) res[rt] = chain(fr[rt], qb);
-            }
-            if (HAS_P2C) {
-                res[3] = chain(fq[0], kb[0]);
-                res[4] = chain(fq[0], kb[1]);
-                if (w & 1) res[5] = chain(fq[1], kb[1]);   // key tile (w & 1): a wave-uniform branch, no register copies
-                else res[5] = chain(fq[1], kb[0]);
+                for (int rt = 0; rt < 2; ++rt) pack_c(chain(fr[rt], qb), cpk[rt]);
             }
         };
-        auto put_results = [&]() {
-            if (HAS_C2P) {
-#pragma unroll
-                for (int rt = 0; rt < 3; ++rt)
-#pragma unroll
-                    for (int a = 0; a < 4; ++a)
-                        *reinterpret_cast<float4*>(&sm.c[w][il * CS + 32 * rt + 8 * a + 4 * hh]) =
-                            float4{res[rt][4 * a], res[rt][4 * a + 1], res[rt][4 * a + 2], res[rt][4 * a + 3]};
-            }
+        auto products_p = [&]() {
             if (HAS_P2C) {
-                auto put_p = [&](int rt, int jt, const f32x16& acc) {
+                pack_p(chain(fq[0], kb[0]), ppk[0]);
+                pack_p(chain(fq[0], kb[1]), ppk[1]);
+                if (w == 0) pack_p(chain(fq[1], kb[1]), ppk[2]);        // wave-uniform branches, no register copies
+                else if (w == 1) pack_p(chain(fq[1], kb[0]), ppk[2]);
+            }
+        };
+        // Ring slot of the group (rt, a) of batch t: key 64t + ckey - 32rt - 8a with ckey = 60 + 4il - 4hh; `phase` is
+        // 64t mod 192.
+        uint16_t* const crow = sm.c + (32 * w + il) * CRS;
+        const int ckey = 60 + 4 * il - 4 * hh;
+        auto put_c = [&](int phase) {
+            if (HAS_C2P) {
+                const int cb = phase + ckey;                    // 56 .. 312
+#pragma unroll
+                for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+                    for (int a = 0; a < 4; ++a) {
+                        const int y = cb - 32 * rt - 8 * a;
+                        const int slot = y >= CRING ? y - CRING : y;
+                        *reinterpret_cast<u32x2*>(crow + slot) = cpk[rt][a];
+                    }
+            }
+        };
+        auto put_p = [&]() {
+            if (HAS_P2C) {
+                auto put1 = [&](int xt, int jt, const u32x2 (&v)[4]) {
 #pragma unroll
                     for (int a = 0; a < 4; ++a)
-                        *reinterpret_cast<u32x2*>(&sm.p[(32 * jt + il) * PS + 32 * rt + 8 * a + 4 * hh]) =
-                            pack4<E>(acc[4 * a], acc[4 * a + 1], acc[4 * a + 2], acc[4 * a + 3]);
+                        *reinterpret_cast<u32x2*>(&sm.p[(32 * jt + il) * PS + 32 * xt + 8 * a + 4 * hh]) = v[a];
                 };
-                put_p(w, 0, res[3]);
-                put_p(w, 1, res[4]);
-                put_p(4 + (w >> 1), w & 1, res[5]);
+                put1(w + 1, 0, ppk[0]);
+                put1(w + 1, 1, ppk[1]);
+                if (w == 0) put1(0, 1, ppk[2]);
+                else if (w == 1) put1(5, 0, ppk[2]);
             }
-            if (HAS_C2P) res[2] = res[0];     // the carried tile of the next step
         };
+        auto next_phase = [](int ph) { return ph == 2 * BN ? 0 : ph + BN; };
 
         // First LDS stage of a tile: keys of steps 0 and 1 and the whole window of step 0 (192 rows of either
         // table), 16 chunks of 16 B per thread.  The delta values come first (dl_win for the window, dl_step for
@@ -636,66 +636,68 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
             dl_step[s1][0] = dl_cold[s1][0];
             dl_step[s1][1] = dl_cold[s1][1];
         }
-        TDB_T_DECL
         phase_barrier();                  // first stage of the first tile is in LDS
         while (true) {
-            TDB_PRESET;
             bind_tables();
-            TDB_PSTAMP(1);
-            // products of step 0; window rows of step 1 (they overwrite rows step 0 is done with); fragments of
-            // step 1; prefetch for half A of step 0
+            // Opening: the c2p batches -2, -1, 0 (window rows w + 128.., w + 64.., w.. of step 0) and the p2c products
+            // of step 0; window rows of step 1 (they overwrite rows step 0 is done with); fragments of step 1.
             const int off1 = prev_off(0);
             dl_next[0] = dl_step[0][0];
             dl_next[1] = dl_step[0][1];
             fetch();                      // window rows of step 1; they arrive under the products of step 0
-            load_frags(0, 0, std::true_type{});
-            products(std::true_type{});
-            put_results();
-            TDB_PSTAMP(2);
-            phase_barrier();              // every position wave has its fragments of step 0
-            TDB_PSTAMP(3);
+            load_fp(0, 0);
+            load_fr(0, w + 2 * BN);
+            products_c();
+            put_c(BN);                    // batch -2: phase (-128) mod 192
+            load_fr(0, w + BN);
+            products_c();
+            put_c(2 * BN);                // batch -1
+            load_fr(0, w);
+            products_c();
+            put_c(0);                     // batch 0
+            products_p();
+            put_p();
+            phase_barrier();              // every position wave has read its fragments of step 0
             store(off1);
             dl_next[0] = dl_step[1][0];
             dl_next[1] = dl_step[1][1];
             fetch();                      // window rows of step 2
             dl_next[0] = dl_step[2][0];
             dl_next[1] = dl_step[2][1];
-            TDB_PSTAMP(4);
             phase_barrier();              // window of step 1 complete
-            TDB_PSTAMP(5);
-            load_frags(off1, 1, std::false_type{});
-            TDB_PSTAMP(6);
+            load_fp(off1, 1);
+            load_fr(off1, w);
             // The tile after this one.  Its delta values are read at the end of the last step but one (when the fragment
             // and result registers are no longer needed); its first LDS stage is read from global memory and written
             // to LDS in half A of the last step, where this role has nothing else to do: after the barrier that ends
             // that half, it is already at the next tile's first position products while the score waves finish the
             // last step.
             const Tile nxt = next_tile(cur);
-            TDB_PSTAMP(7);
 
             int off2 = prev_off(off1);    // ring offset of step s+2
+            int phase = BN;               // ring phase of batch s+1
             auto pos_step = [&](int s, auto tail_tag) {
                 constexpr bool TAIL = decltype(tail_tag)::value;   // step nsteps-2: no step s+2 to prepare
-                phase_barrier();          // scratch of step s complete
-                TDB_STAMP(0);
-                products(std::false_type{});   // of step s+1, into registers; issued first: the wait for the
+                phase_barrier();          // position terms of step s complete
+                products_c();             // of step s+1, into registers; issued first: the wait for the
                 __builtin_amdgcn_sched_barrier(0);  // prefetched global data then passes under the MFMAs
                 if (!TAIL) {
                     store(off2);          // new window rows of step s+2
                     fetch();              // window rows of step s+3: a full step ahead of their store
                     fetch_delta(s + 4);
                 }
-                TDB_STAMP(1);
-                phase_barrier();          // score waves are done with the scratch; the staged tiles are visible
-                TDB_STAMP(2);
-                put_results();            // of step s+1
+                phase_barrier();          // score waves are done with the ring slots and the scratch; the staged tiles are visible
+                put_c(phase);             // of step s+1
+                products_p();             // of step s+1: the matrix pipe is shared with the score wave's P.V in this half,
+                put_p();                  // with its S^T in the other
                 if (!TAIL) {
-                    load_frags(off2, s & 1, std::false_type{});  // of step s+2
+                    load_fp(off2, s & 1); // of step s+2
+                    load_fr(off2, w);
                 } else {
                     read_deltas(nxt);
                 }
                 off2 = prev_off(off2);
-                TDB_STAMP(3);
+                phase = next_phase(phase);
             };
             if (nsteps >= 2) {
                 for (int s = 0; s + 2 < nsteps; ++s) pos_step(s, std::false_type{});
@@ -703,23 +705,18 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
             } else {
                 read_deltas(nxt);
             }
-            // Last key step: nothing left to prepare for this tile.  The ring, both key buffers and the Q fragment
+            // Last key step: nothing left to prepare for this tile.  The rings, both key buffers and the Q fragment
             // registers are free, so the next tile moves in; the barrier that ends this half is also the barrier
             // after which the next tile's first stage is in LDS.
             phase_barrier();
-            TDB_STAMP(0);
             read_stage(nxt);
             load_q(qb, nxt);              // (the last products of this tile have read the old fragments)
             if (nxt.vb >= 0) write_stage();
-            TDB_STAMP(1);
             phase_barrier();
-            TDB_STAMP(2);
             if (nxt.vb < 0) break;
             cur = nxt;
             bind(cur);
         }
-        TDB_T_FLUSH(6);
-        TDB_P_FLUSH;
         return;
     }
 
@@ -735,6 +732,13 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
 #pragma unroll
             for (int c = 0; c < 4; ++c) kf[jt][c] = lds_frag<X8>(sm.k[kbuf], 32 * jt + il, 16 * c + 8 * hh);
     };
+    // Identity fragments: A operand that adds a B operand of 16 keys x 32 queries onto rows 16c2 .. 16c2+15 of a score
+    // tile.  Lane (row il, half hh) of an A operand holds columns 8hh .. 8hh+7 of its row.
+    X8 idf[2];
+#pragma unroll
+    for (int c2 = 0; c2 < 2; ++c2)
+#pragma unroll
+        for (int t = 0; t < 8; ++t) idf[c2][t] = il == 16 * c2 + 8 * hh + t ? (ET)1.0f : (ET)0.0f;
     // Keys and values travel global -> registers -> LDS through the score waves: thread tid stages chunk sch of rows
     // srow and srow + 32 of a 64-row step.  Buffer loads: the buffer of a step starts at its first row and ends with
     // the last row of the sequence, so rows past the end come back as zeros (hardware range check) with no lane
@@ -769,67 +773,61 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     };
     Tile nxt;                             // the tile after the current one (looked up while a tile opens)
     nxt.vb = -1;
-    nxt.head = nxt.b = nxt.row0 = nxt.len = nxt.cost = 0;
+    nxt.head = nxt.b = nxt.row0 = nxt.len = 0;
+    nxt.cost = 0;
     nxt.tok0 = 0;
-    TDB_T_DECL
+    int cphase = 0;                       // ring slot of the first key of the step: 64s mod 192
+    const uint16_t* const crow = sm.c + (32 * w + il) * CRS + 8 * hh;
     // One key step.  MASKED: the step reaches past the end of the sequence (only the last step can).
     auto key_step = [&](int s, auto masked_tag) {
         constexpr bool MASKED = decltype(masked_tag)::value;
-        phase_barrier();                  // scratch of step s complete
-        TDB_STAMP(0);
+        phase_barrier();                  // position terms of step s complete
 
         // ---- half A: keys of step s+2 and values of step s go to LDS (prefetched registers, nothing waits);
-        //      position terms of step s out of the scratch.  Element (jj, i) of the score tile takes
-        //      C'[i][i-jj+63] (fp32, straight into the accumulator) and P'[jj][32w+i-jj+63] (bf16) ----------------
+        //      position terms of step s: c2p as four B operands of 16 keys each, straight out of the ring (keys
+        //      64s .. 64s+63 never straddle its wrap), p2c element by element: (key jj, query n) takes
+        //      P'[jj][w + 4n + 63 - jj], converted to fp32 into what becomes the initial score accumulator ----------
         store_kv(s & 1, s + 2 < nsteps);  // (in the last step the key buffers already take the next tile's keys)
-        // The gathers are ordinary LDS loads of dwords at 4-byte alignment; the compiler pairs them into two-address
-        // reads and places the waits.  (Loads issued from inline assembly would be invisible to it: it may then copy
-        // a destination register before the data has arrived.)
-        f32x16 s_acc[2];
+        X8 cf[2][2];
         if (HAS_C2P) {
-            // float index of element e of key tile jt:  il*CS + il + 63 - 4*hh - jc,  jc = 32*jt + 8*(e>>2) + (e&3) <= 59
-            const auto* cbase = TDB_LDS(const float, &sm.c[w][il * (CS + 1) + 4 - 4 * hh]);
 #pragma unroll
             for (int jt = 0; jt < 2; ++jt)
 #pragma unroll
-                for (int e = 0; e < 16; ++e) s_acc[jt][e] = cbase[59 - (32 * jt + 8 * (e >> 2) + (e & 3))];
+                for (int c2 = 0; c2 < 2; ++c2) cf[jt][c2] = *reinterpret_cast<const X8*>(crow + cphase + 32 * jt + 16 * c2);
+        }
+        f32x16 s_acc[2];
+        if (HAS_P2C) {
+            // The gathers are ordinary LDS loads; the compiler places the waits.  (Loads issued from inline assembly
+            // would be invisible to it: it may then copy a destination register before the data has arrived.)
+            const auto* pbase = TDB_LDS(const uint16_t, sm.p) + (w + 63 + 4 * il) + 4 * hh * (PS - 1);
+#pragma unroll
+            for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) s_acc[jt][e] = E::widen(pbase[(32 * jt + 8 * (e >> 2) + (e & 3)) * (PS - 1)]);
         } else {
             s_acc[0] = zero16;
             s_acc[1] = zero16;
         }
-        if (HAS_P2C) {
-            // Element (key j, query il) is P'[j][X - j], X = 32w + il + 63: from one key to the next the bf16 index moves
-            // by PS - 1 (odd), so the element alternates between the low and the high half of its dword with the
-            // parity of j, starting from the parity of il.  The dwords of keys j and j + 2 are (PS - 1) dwords apart
-            // (one two-address read); a byte permute with a per-lane selector moves the wanted half into an fp32.
-            constexpr int PD = PS - 1;            // dwords between the elements of keys j and j + 2
-            const int X = 32 * w + il + 63, pl = X & 1;
-            const auto* pbase = TDB_LDS(const uint32_t, sm.p) + (X - pl) / 2 + 2 * hh * PD;   // dword of element (4hh, X - 4hh)
-            const uint32_t sel_even = pl ? E::PICK_HI : E::PICK_LO, sel_odd = pl ? E::PICK_LO : E::PICK_HI;
-            uint32_t g[2][16];
-#pragma unroll
-            for (int jt = 0; jt < 2; ++jt)
-#pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    const int jc = 32 * jt + 8 * (e >> 2) + (e & 3);
-                    g[jt][e] = (jc & 1) ? pbase[pl + (jc * PD - 1) / 2] : pbase[(jc / 2) * PD];
-                }
-#pragma unroll
-            for (int jt = 0; jt < 2; ++jt)
-#pragma unroll
-                for (int e = 0; e < 16; ++e)
-                    s_acc[jt][e] += E::pick(g[jt][e], (e & 1) ? sel_odd : sel_even);
-        }
-        TDB_STAMP(1);
-        phase_barrier();                  // scratch is free again; keys of step s+1 and values of step s are staged
-        TDB_STAMP(2);
-
-        // ---- half B ---------------------------------------------------------------------------------------------
+        cphase = cphase == 2 * BN ? 0 : cphase + BN;
+        // all LDS reads of the half in flight together, then the conversions, then the score MFMAs (they share the
+        // matrix pipe of this half with the position wave of the SIMD)
+        __builtin_amdgcn_sched_group_barrier(0x200, 4, 0);    // K / V stores
+        __builtin_amdgcn_sched_group_barrier(0x100, 36, 0);   // ring fragments and P' elements
+        __builtin_amdgcn_sched_group_barrier(0x002, 32, 0);   // conversions
 #pragma unroll
         for (int c = 0; c < 4; ++c)
 #pragma unroll
             for (int jt = 0; jt < 2; ++jt) s_acc[jt] = E::mfma(kf[jt][c], qb[c], s_acc[jt]);
-        load_kf((s + 1) & 1);             // K fragments of step s+1 (the MFMAs above have read this step's)
+        if (HAS_C2P) {
+#pragma unroll
+            for (int c2 = 0; c2 < 2; ++c2)
+#pragma unroll
+                for (int jt = 0; jt < 2; ++jt) s_acc[jt] = E::mfma(idf[c2], cf[jt][c2], s_acc[jt]);
+        }
+        if (s + 1 < nsteps) load_kf((s + 1) & 1);   // K fragments of step s+1 (the MFMAs above have read this step's)
+        phase_barrier();                  // ring slots and scratch are free again; keys of step s+1 and values of step s are staged
+
+        // ---- half B ---------------------------------------------------------------------------------------------
         if (s + 1 == nsteps) load_q(qb, nxt);   // last step: the Q fragments of the next tile travel from here on
         if (s + 1 < nsteps) fetch_kv(s + 3, s + 1);   // for the next half A (nothing left to fetch in the last step)
         // V^T fragments through the transposing LDS read: the lane provides the address of 4 dims of one key
@@ -859,7 +857,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
                     if (j >= len) s_acc[jt][e] = -INFINITY;
                 }
         }
-        // streaming softmax: this lane holds 32 of the 64 keys of query row il, lane^32 the others
+        // streaming softmax: this lane holds 32 of the 64 keys of its query row, lane^32 the others
         float mx = s_acc[0][0];
 #pragma unroll
         for (int jt = 0; jt < 2; ++jt)
@@ -901,7 +899,6 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
                     o_acc[dt] = E::mfma(vf[jt][c][dt], pb, o_acc[dt]);
             }
         l_run += psum;
-        TDB_STAMP(3);
     };
 
     // Opening of a tile, after its first barrier (first stage in LDS).  Everything that reads global memory is
@@ -912,30 +909,25 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     uint16_t* o_ptr = nullptr;
     bool o_write = false;
     auto open_tile = [&]() {
-        TDB_PRESET;
         load_kf(0);
         fetch_kv(2, 0);
-        TDB_PSTAMP(0);
         if (o_write) {
 #pragma unroll
             for (int dt = 0; dt < 2; ++dt)
 #pragma unroll
                 for (int a = 0; a < 2; ++a) *reinterpret_cast<u32x4*>(o_ptr + 32 * dt + 16 * a) = o_out[dt][a];
         }
-        TDB_PSTAMP(3);
+        cphase = 0;
         phase_barrier();                  // the two opening barriers of the position waves
-        TDB_PSTAMP(4);
         phase_barrier();
-        TDB_PSTAMP(5);
         // the tile after this one is looked up while the position waves get step 1 ready
         nxt = next_tile(cur);
-        TDB_PSTAMP(1);
     };
-    // Epilogue of a tile: normalised output rows, packed.  A lane holds d = 32*dt + 8*a + 4*hh + 0..3 of query row il,
+    // Epilogue of a tile: normalised output rows, packed.  A lane holds d = 32*dt + 8*a + 4*hh + 0..3 of its query row,
     // its partner lane^32 the other four of every eight; one swap between the lane halves per dword gives each lane
     // eight consecutive d (lane half hh keeps the blocks a = 2*a2 + hh), so a row goes out in 16-byte stores.
     auto close_tile = [&]() {
-        const int qi = row0 + 32 * w + il;
+        const int qi = row0 + 4 * il + w;
         const float l_tot = l_run + __shfl_xor(l_run, 32);
         const float inv = 1.f / l_tot;
         const bool live = qi < len;
@@ -950,7 +942,8 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
                 for (int t = 0; t < 2; ++t) {
                     const int a = 2 * a2 + t;
                     r[t] = u32x2{0, 0};
-                    if (live) r[t] = pack4<E>(o_acc[dt][4 * a] * inv, o_acc[dt][4 * a + 1] * inv, o_acc[dt][4 * a + 2] * inv, o_acc[dt][4 * a + 3] * inv);
+                    if (live) r[t] = u32x2{pack2<E>(o_acc[dt][4 * a] * inv, o_acc[dt][4 * a + 1] * inv),
+                                           pack2<E>(o_acc[dt][4 * a + 2] * inv, o_acc[dt][4 * a + 3] * inv)};
                 }
                 // lower half: (own block 2*a2, partner's block 2*a2); upper half: (partner's block 2*a2+1, own block 2*a2+1)
                 const auto k0 = __builtin_amdgcn_permlane32_swap(r[0][0], r[1][0], false, false);
@@ -971,10 +964,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
 
         // The position waves put the first stage of the next tile into LDS during the last step and are at its
         // first position products by now; this tile is closed under those.
-        TDB_PRESET;
         close_tile();
-        TDB_PSTAMP(7);
-        TDB_STAMP(5);
         if (nxt.vb < 0) break;
         cur = nxt;
         bind(cur);
@@ -986,9 +976,6 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
 #pragma unroll
             for (int a = 0; a < 2; ++a) *reinterpret_cast<u32x4*>(o_ptr + 32 * dt + 16 * a) = o_out[dt][a];
     }
-    TDB_T_FLUSH(0);
-    TDB_P_FLUSH;
-    TDB_TRACE_EXIT;
 }
 
 }  // namespace
@@ -1004,6 +991,18 @@ bool tdb_mfma_supported(const TdbKernelParams& p, int dtype) {
     if (p.pq && int64_t(2) * p.span * p.pqs_r * 2 >= lim) return false;
     return true;
 }
+
+namespace {
+
+// Per-device launch facts, looked up once per device under a lock: CU count (rounded down to the 8 XCDs the block
+// ids are dealt over) and, per kernel instance, whether its dynamic-LDS limit has been raised on that device.
+constexpr int kMaxDevices = 64;
+constexpr int kInstances = 8;
+std::mutex g_dev_mutex;
+int g_cus[kMaxDevices] = {0};
+bool g_attr_set[kMaxDevices][kInstances] = {{false}};
+
+}  // namespace
 
 hipError_t tdb_launch_mfma(const TdbKernelParams& whole, int dtype, hipStream_t stream) {
     // Packed batches of more than 64 sequences go out as several launches of at most 64 (even parts): the kernel
@@ -1025,42 +1024,44 @@ hipError_t tdb_launch_mfma(const TdbKernelParams& whole, int dtype, hipStream_t 
     const int64_t tiles = int64_t(p.varlen ? p.total / BM + p.B : p.B * ((p.L + BM - 1) / BM)) * p.H;
     const int64_t round = 8 * XCD_GROUP;                 // the id regrouping is a bijection on multiples of this
     const int nblocks = int((tiles + round - 1) / round * round);
-    // persistent workgroups: one per CU, in multiples of the 8 XCDs the ids are dealt over
-    static int cus_of[64] = {0};
     int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
-    if (cus_of[dev] == 0) {
-        int n = 0;
-        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 8) n = 8;
-        cus_of[dev] = n / 8 * 8;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+    const bool c2p = p.pk != nullptr, p2c = p.pq != nullptr;
+    const int instance = (dtype == TDB_F16 ? 4 : 0) + (c2p ? 2 : 0) + (p2c ? 1 : 0);
+    const size_t smem = sizeof(Smem);
+    const void* fn = nullptr;
+#define TDB_PICK(A, B, T) fn = reinterpret_cast<const void*>(&attn_mfma_kernel<A, B, T>)
+#define TDB_PICK_T(T)                                      \
+    do {                                                   \
+        if (c2p && p2c) TDB_PICK(true, true, T);           \
+        else if (c2p) TDB_PICK(true, false, T);            \
+        else if (p2c) TDB_PICK(false, true, T);            \
+        else TDB_PICK(false, false, T);                    \
+    } while (0)
+    if (dtype == TDB_F16) TDB_PICK_T(TDB_F16);
+    else TDB_PICK_T(TDB_BF16);
+#undef TDB_PICK_T
+#undef TDB_PICK
+    int cus = 0;
+    {
+        std::lock_guard<std::mutex> lock(g_dev_mutex);
+        if (g_cus[dev] == 0) {
+            int n = 0;
+            if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 8) n = 8;
+            g_cus[dev] = n / 8 * 8;
+        }
+        cus = g_cus[dev];
+        if (!g_attr_set[dev][instance]) {
+            e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, int(smem));
+            if (e != hipSuccess) return e;
+            g_attr_set[dev][instance] = true;
+        }
     }
     // Persistent workgroups, one per CU: fixed layout with a strided deal (tiles cost about the same), packed
     // batches with a cost-balanced deal computed in the kernel.
-    const int persistent = nblocks < cus_of[dev] ? nblocks : cus_of[dev];
-    const dim3 grid{unsigned(persistent)}, block(NTHREADS);
-    const size_t smem = sizeof(Smem);
-    const bool c2p = p.pk != nullptr, p2c = p.pq != nullptr;
-#define TDB_LAUNCH(A, B, T)                                                                                     \
-    do {                                                                                                        \
-        static bool attr_set = false;                                                                           \
-        if (!attr_set) {                                                                                        \
-            (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_mfma_kernel<A, B, T>),                \
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, int(smem));                   \
-            attr_set = true;                                                                                    \
-        }                                                                                                       \
-        hipLaunchKernelGGL((attn_mfma_kernel<A, B, T>), grid, block, smem, stream, p, nblocks);                 \
-    } while (0)
-#define TDB_LAUNCH_T(T)                                                                                         \
-    do {                                                                                                        \
-        if (c2p && p2c) TDB_LAUNCH(true, true, T);                                                              \
-        else if (c2p) TDB_LAUNCH(true, false, T);                                                               \
-        else if (p2c) TDB_LAUNCH(false, true, T);                                                               \
-        else TDB_LAUNCH(false, false, T);                                                                       \
-    } while (0)
-    if (dtype == TDB_F16) TDB_LAUNCH_T(TDB_F16);
-    else TDB_LAUNCH_T(TDB_BF16);
-#undef TDB_LAUNCH_T
-#undef TDB_LAUNCH
-    return hipGetLastError();
+    const int persistent = nblocks < cus ? nblocks : cus;
+    void* args[] = {const_cast<TdbKernelParams*>(&p), const_cast<int*>(&nblocks)};
+    return hipLaunchKernel(fn, dim3(unsigned(persistent)), dim3(NTHREADS), args, smem, stream);
 }
-
