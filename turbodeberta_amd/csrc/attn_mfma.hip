@@ -351,12 +351,10 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     // role leans on the LDS and the other on the matrix cores:
     //   A  score waves read this step's position terms (c2p ring fragments, P' scratch), hand register-prefetched
     //      keys (step s+2) and values (step s) to LDS, run the S^T(s) MFMAs on top of the position terms and pick up
-    //      the K fragments of step s+1; position waves run the c2p MFMAs of step s+1 on fragments they already hold,
-    //      then store the 64 new window rows of step s+2 and request those of step s+3;
+    //      the K fragments of step s+1; position waves run the position MFMAs of step s+1 on fragments they already
+    //      hold, then store the 64 new window rows of step s+2 and request those of step s+3;
     //   B  score waves: softmax(s), P.V(s), and they request keys and values for the next half A; position waves:
-    //      c2p results of step s+1 into the ring, the p2c MFMAs of step s+1 and their results into the now free
-    //      scratch, LDS fragments of step s+2.
-    // (Each half so carries half of the step's MFMAs and half of its LDS traffic.)
+    //      results of step s+1 into the ring and the now free scratch, LDS fragments of step s+2.
     // Both roles pass 2 + 2*nsteps barriers per tile (the barrier that ends the last step is also the one after which
     // the next tile's first stage is visible) and walk the same tile list.
     //
@@ -680,6 +678,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
                 constexpr bool TAIL = decltype(tail_tag)::value;   // step nsteps-2: no step s+2 to prepare
                 phase_barrier();          // position terms of step s complete
                 products_c();             // of step s+1, into registers; issued first: the wait for the
+                products_p();
                 __builtin_amdgcn_sched_barrier(0);  // prefetched global data then passes under the MFMAs
                 if (!TAIL) {
                     store(off2);          // new window rows of step s+2
@@ -688,8 +687,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
                 }
                 phase_barrier();          // score waves are done with the ring slots and the scratch; the staged tiles are visible
                 put_c(phase);             // of step s+1
-                products_p();             // of step s+1: the matrix pipe is shared with the score wave's P.V in this half,
-                put_p();                  // with its S^T in the other
+                put_p();
                 if (!TAIL) {
                     load_fp(off2, s & 1); // of step s+2
                     load_fr(off2, w);
