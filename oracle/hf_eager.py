@@ -10,14 +10,15 @@ and only as the checker.
 Pin status of each function (what independent evidence fixes it):
 
 * ``log_bucket_position`` / ``relative_position_index`` -- pinned: closed-form zones, spot
-  values, antisymmetry/monotonicity, a float64 margin proof, a C restatement
-  (``oracle/bucket_ref.c``) and a golden table written by HF's own
+  values, antisymmetry/monotonicity, a float64 margin proof, a float64 scalar restatement
+  (``bucket_scalar`` below) and golden tables written by HF's own
   ``make_log_bucket_position`` (``tests/golden/hf_bucket_table.npz``).
 * ``disentangled_bias`` / ``attention`` -- pinned: brute-force triple loop on tiny shapes,
   Toeplitz invariant, reduction to ``torch.nn.functional.scaled_dot_product_attention`` when
   the position terms vanish, and golden outputs written by HF's
-  ``DisentangledSelfAttention.forward`` (``tests/golden/hf_layer_*.npz``).
-* ``self_attention_layer`` -- pinned by the same HF golden outputs (config-1 layer).
+  ``DisentangledSelfAttention.forward`` (``tests/golden/hf_layer_outputs.npz``).
+* ``self_attention_layer`` -- pinned by the same HF golden outputs (config-1 layer);
+  a two-layer model output is in ``tests/golden/hf_tiny_model.npz``.
 * ``encoder_attention_mask`` -- pinned by an HF golden 2x8 toy
   (``tests/golden/hf_mask_toy.npz``).
 """

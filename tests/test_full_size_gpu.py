@@ -137,6 +137,66 @@ def test_config5_long_context_l4096():
     assert_close_bf16(outv[s:e].permute(1, 0, 2), ref1, "config 5 packed", tol=1e-2)
 
 
+def test_config5_stated_shape_b4_h12_l4096():
+    """BASELINE config 5 at its stated shape (batch 4 x 12 heads x seq 4096, full mask): every workgroup walks many
+    tiles of 64 key steps, most of them far beyond max_relative_positions.  Whole tensor: the packed run of the same
+    tokens is bit-identical; head subset: the vector-ALU kernel agrees within bf16 rounding; one (sequence, 2 heads):
+    the CPU oracle."""
+    B, L = 4, 4096
+    q, k, v, pk, pq = _projected(B, L, seed=7)
+    print("[case] config 5 stated shape, fixed", flush=True)
+    out = flash_attention_with_disentangled(q, k, v, None, None, False, SCALE, BUCKETS, MAX_REL,
+                                            pos_key_layer=pk, pos_query_layer=pq)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out.float()).all()
+    tok = lambda t: t.permute(0, 2, 1, 3).reshape(B * L, H, D)             # [T, H, D] view of the same storage
+    cu = torch.arange(B + 1, dtype=torch.int32, device=DEV) * L
+    print("[case] config 5 stated shape, packed", flush=True)
+    outv = flash_attention_with_disentangled_varlen(tok(q), tok(k), tok(v), None, None, cu, cu, L, L, False, SCALE,
+                                                    BUCKETS, MAX_REL, pos_key_layer=pk, pos_query_layer=pq)
+    assert torch.equal(outv, tok(out))
+    hs = [0, 7, 11]
+    print("[case] config 5 stated shape, vector-ALU kernel on 3 heads of sequence 2", flush=True)
+    sub = lambda t: t[2:3, hs]
+    gen = flash_attention_with_disentangled(sub(q), sub(k), sub(v), None, None, False, SCALE, BUCKETS, MAX_REL,
+                                            pos_key_layer=pk[hs], pos_query_layer=pq[hs], force_generic=True)
+    assert (out[2:3, hs].float() - gen.float()).abs().max().item() <= 1e-2
+    hs = [3, 8]
+    f = lambda t: t[1:2, hs].float().cpu()
+    ref = O.attention(f(q), f(k), f(v), pk[hs].float().cpu(), pq[hs].float().cpu(), None,
+                      position_buckets=BUCKETS, max_relative_positions=MAX_REL)
+    assert_close_bf16(out[1:2, hs], ref, "config 5 stated shape vs oracle", tol=1e-2)
+
+
+def test_config5_packed_variant_8_sequences():
+    """BASELINE config 5, packed variant: 8 sequences with lengths uniform in [1024, 4096] (seed 0), 12 heads.  Every
+    sequence on its own through the fixed-length operator is bit-identical; the shortest sequence, 2 heads, against
+    the CPU oracle."""
+    lengths = np.random.RandomState(0).randint(1024, 4097, size=8)
+    T = int(lengths.sum())
+    q, k, v, pk, pq = _projected(1, T, seed=9)
+    tok = lambda t: t[0].permute(1, 0, 2)
+    cu_np = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    cu = torch.from_numpy(cu_np).to(DEV)
+    print(f"[case] config 5 packed variant, lengths {lengths.tolist()}", flush=True)
+    out = flash_attention_with_disentangled_varlen(tok(q), tok(k), tok(v), None, None, cu, cu, 4096, 4096, False, SCALE,
+                                                   BUCKETS, MAX_REL, pos_key_layer=pk, pos_query_layer=pq)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out.float()).all()
+    for b in range(8):
+        s, e = int(cu_np[b]), int(cu_np[b + 1])
+        one = flash_attention_with_disentangled(q[:, :, s:e], k[:, :, s:e], v[:, :, s:e], None, None, False, SCALE,
+                                                BUCKETS, MAX_REL, pos_key_layer=pk, pos_query_layer=pq)
+        assert torch.equal(one[0].permute(1, 0, 2), out[s:e]), b
+    b = int(lengths.argmin())
+    s, e = int(cu_np[b]), int(cu_np[b + 1])
+    hs = [1, 10]
+    f = lambda t: t[:, hs, s:e].float().cpu()
+    ref = O.attention(f(q), f(k), f(v), pk[hs].float().cpu(), pq[hs].float().cpu(), None,
+                      position_buckets=BUCKETS, max_relative_positions=MAX_REL)[0]
+    assert_close_bf16(out[s:e][:, hs].permute(1, 0, 2), ref, "config 5 packed variant vs oracle", tol=1e-2)
+
+
 def test_persistent_tile_walk_mixed_lengths():
     """More tiles than workgroups, with everything a persistent workgroup can meet on its list: single-step tiles
     (length <= 64), tiles with only padded rows (in the middle and at the end of a list), a sequence of length 0,

@@ -314,3 +314,204 @@ def test_query_states_from_another_tensor():
         got = ours(hidden, mask4, False, query_states=queries, rel_embeddings=rel)[0]
     valid = mask2.bool()
     assert (got[valid] - want[valid]).abs().max().item() <= 1e-4 * want[valid].abs().max().item()
+
+
+def _pair(cls_name, cfg, seed, flash_name=None):
+    """(ours, theirs) on the GPU, fp32, eval: the Hugging Face class and the fused class of the same name with the
+    same seeded parameters."""
+    import transformers.models.deberta_v2.modeling_deberta_v2 as hf
+    from turbodeberta_amd import model as fused
+    theirs = getattr(hf, "DebertaV2" + cls_name)(cfg).eval()
+    fill_params(theirs, seed=seed)
+    ours = getattr(fused, flash_name or ("FlashDebertaV2" + cls_name))(cfg).eval()
+    ours.load_state_dict(theirs.state_dict())
+    return ours.to("cuda:0"), theirs.to("cuda:0")
+
+
+@pytest.mark.gpu
+def test_masked_lm_matches_hf_eager():
+    """FlashDebertaV2ForMaskedLM (reference model.py:244-262): logits over the vocabulary on valid tokens."""
+    cfg = _tiny()
+    ours, theirs = _pair("ForMaskedLM", cfg, seed=31)
+    ids, mask = tiny_model_inputs()
+    ids, mask = torch.from_numpy(ids).cuda(), torch.from_numpy(mask).cuda()
+    print("[case] masked LM head", flush=True)
+    with torch.no_grad():
+        a = ours(input_ids=ids, attention_mask=mask).logits
+        b = theirs(input_ids=ids, attention_mask=mask).logits
+    valid = mask.bool()
+    assert a.shape == b.shape == (*ids.shape, cfg.vocab_size)
+    assert (a[valid] - b[valid]).abs().max().item() <= 1e-4 * b[valid].abs().max().item()
+
+
+@pytest.mark.gpu
+def test_question_answering_matches_hf_eager():
+    """FlashDebertaV2ForQuestionAnswering (reference model.py:290-301): start / end logits on valid tokens."""
+    cfg = DebertaV2Config(**dict(tiny_model_config(), num_labels=2))
+    ours, theirs = _pair("ForQuestionAnswering", cfg, seed=32)
+    ids, mask = tiny_model_inputs()
+    ids, mask = torch.from_numpy(ids).cuda(), torch.from_numpy(mask).cuda()
+    print("[case] question answering head", flush=True)
+    with torch.no_grad():
+        a = ours(input_ids=ids, attention_mask=mask)
+        b = theirs(input_ids=ids, attention_mask=mask)
+    valid = mask.bool()
+    for x, y in ((a.start_logits, b.start_logits), (a.end_logits, b.end_logits)):
+        assert x.shape == y.shape == tuple(ids.shape)
+        assert (x[valid] - y[valid]).abs().max().item() <= 1e-4 * y[valid].abs().max().item()
+
+
+@pytest.mark.gpu
+def test_multiple_choice_matches_hf_eager():
+    """FlashDebertaV2ForMultipleChoice (reference model.py:303-314): ids [batch, choices, L]; one logit per choice."""
+    cfg = _tiny()
+    ours, theirs = _pair("ForMultipleChoice", cfg, seed=33)
+    rs = np.random.RandomState(5)
+    B, C, L = 2, 3, 24
+    lens = rs.randint(1, L + 1, size=(B, C))
+    mask = torch.from_numpy((np.arange(L)[None, None] < lens[:, :, None]).astype(np.int64)).cuda()
+    ids = torch.from_numpy(rs.randint(1, cfg.vocab_size, size=(B, C, L))).cuda() * mask
+    print("[case] multiple choice head", flush=True)
+    with torch.no_grad():
+        a = ours(input_ids=ids, attention_mask=mask).logits
+        b = theirs(input_ids=ids, attention_mask=mask).logits
+    assert a.shape == b.shape == (B, C)
+    assert (a - b).abs().max().item() <= 1e-4 * b.abs().max().item()
+
+
+@pytest.mark.gpu
+def test_enhanced_mask_decoder_step():
+    """The body of the ``z_steps > 1`` loop (modeling_deberta_v2.py:772-788): the last layer run again with the previous
+    output as ``query_states``, the encoder's 4-D mask, its relative-position matrix and relative embeddings.  (The loop
+    itself cannot run in transformers 5.15 -- it appends to a tuple -- for the eager model either, which this test
+    records; the layer call it makes is compared directly.)"""
+    cfg = _tiny()
+    ours, theirs = _pair("Model", cfg, seed=34)
+    ids, mask = tiny_model_inputs()
+    ids, mask = torch.from_numpy(ids).cuda(), torch.from_numpy(mask).cuda()
+    print("[case] enhanced mask decoder step", flush=True)
+    with torch.no_grad():
+        enc = theirs(input_ids=ids, attention_mask=mask, output_hidden_states=True)
+        hidden, queries = enc.hidden_states[-2], enc.hidden_states[-1]
+        rel = theirs.encoder.get_rel_embedding()
+        mask4 = theirs.encoder.get_attention_mask(mask)
+        rel_pos = theirs.encoder.get_rel_pos(hidden)
+        want = theirs.encoder.layer[-1](hidden, mask4, output_attentions=False, query_states=queries,
+                                        relative_pos=rel_pos, rel_embeddings=rel)[0]
+        got = ours.encoder.layer[-1](hidden, mask4, output_attentions=False, query_states=queries,
+                                     relative_pos=rel_pos, rel_embeddings=ours.encoder.get_rel_embedding())[0]
+        theirs.z_steps = 2
+        with pytest.raises(AttributeError):                                   # Hugging Face's own loop is dead code
+            theirs(input_ids=ids, attention_mask=mask)
+    valid = mask.bool()
+    assert (got[valid] - want[valid]).abs().max().item() <= 1e-4 * want[valid].abs().max().item()
+    assert (want[valid] - queries[valid]).abs().max().item() > 1e-3          # the step does something
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("buckets", [-1, 0])
+def test_model_without_log_buckets(buckets):
+    """``position_buckets <= 0``: plain clamped relative positions, span = max_relative_positions
+    (modeling_deberta_v2.py:170-176, :585-588)."""
+    cfg = DebertaV2Config(**dict(tiny_model_config(), position_buckets=buckets, max_relative_positions=24))
+    ours, theirs = _pair("Model", cfg, seed=35)
+    ids, mask = tiny_model_inputs()                                             # L = 40 > max_relative_positions
+    ids, mask = torch.from_numpy(ids).cuda(), torch.from_numpy(mask).cuda()
+    print(f"[case] model with position_buckets={buckets}", flush=True)
+    with torch.no_grad():
+        a = ours(input_ids=ids, attention_mask=mask).last_hidden_state
+        b = theirs(input_ids=ids, attention_mask=mask).last_hidden_state
+    valid = mask.bool()
+    assert (a[valid] - b[valid]).abs().max().item() <= 1e-4 * b[valid].abs().max().item()
+
+
+@pytest.mark.gpu
+def test_inference_mode_padded_and_unpadded():
+    """Under ``torch.inference_mode()`` masks are inference tensors without a modification counter; both the packed
+    path (batch with padding) and the padded path (batch without) must run and agree with ``no_grad``."""
+    cfg = _tiny()
+    ours, theirs = _pair("Model", cfg, seed=36)
+    ids, mask = tiny_model_inputs()
+    ids, mask = torch.from_numpy(ids).cuda(), torch.from_numpy(mask).cuda()
+    full = torch.ones_like(mask)
+    print("[case] inference mode", flush=True)
+    with torch.no_grad():
+        want_pad = theirs(input_ids=ids, attention_mask=mask).last_hidden_state
+        want_full = theirs(input_ids=ids, attention_mask=full).last_hidden_state
+    with torch.inference_mode():
+        got_pad = ours(input_ids=ids, attention_mask=mask).last_hidden_state
+        got_full = ours(input_ids=ids, attention_mask=full).last_hidden_state
+        again = ours(input_ids=ids.clone(), attention_mask=mask.clone()).last_hidden_state   # masks created inside
+    valid = mask.bool()
+    assert (got_pad[valid] - want_pad[valid]).abs().max().item() <= 1e-4 * want_pad[valid].abs().max().item()
+    assert (got_full - want_full).abs().max().item() <= 1e-4 * want_full.abs().max().item()
+    assert torch.equal(again, got_pad)
+
+
+@pytest.mark.gpu
+def test_masks_that_are_not_right_padded_raise():
+    """Left padding, holes and a 4-D mask that is not ``m_i * m_j`` cannot be expressed as per-sequence lengths: the
+    fused paths refuse them instead of attending to the wrong tokens (eager Hugging Face handles them)."""
+    cfg = _tiny()
+    ours, _ = _pair("Model", cfg, seed=37)
+    ids, mask = tiny_model_inputs()
+    ids, mask = torch.from_numpy(ids).cuda(), torch.from_numpy(mask).cuda()
+    left = torch.flip(mask, dims=[1])
+    holes = mask.clone()
+    holes[0, 5] = 0
+    for bad in (left, holes):
+        for pack in (True, False):
+            ours.encoder.pack_sequences = pack
+            with torch.no_grad(), pytest.raises(ValueError, match="right padded"):
+                ours(input_ids=ids, attention_mask=bad)
+    ours.encoder.pack_sequences = True
+    att = ours.encoder.layer[0].attention.self
+    hidden = torch.randn(3, 40, cfg.hidden_size, device="cuda:0")
+    rel = ours.encoder.get_rel_embedding()
+    ext = mask.unsqueeze(1).unsqueeze(2)
+    m4 = (ext * ext.squeeze(-2).unsqueeze(-1)).clone()
+    m4[0, 0, 3, 7] = 0                                                          # a real [L, L] pattern
+    with torch.no_grad(), pytest.raises(ValueError, match="right padded"):
+        att(hidden, m4, False, rel_embeddings=rel)
+
+
+@pytest.mark.gpu
+def test_config4_v3_large_encoder_b16_l512():
+    """BASELINE config 4 at its stated shape: 24 layers x 1024, 16 heads x 64, FFN 4096, vocabulary 128100, buckets 256,
+    max_rel 512, random N(0, 0.02) weights, bf16; ids [16, 512] with valid lengths uniform in [64, 512].  The patched
+    model (reference model.py:204-242), packed and padded, must be as close to the float32 Hugging Face model on the
+    same device as Hugging Face's own bf16 eager run is."""
+    cfg = DebertaV2Config(vocab_size=128100, hidden_size=1024, num_hidden_layers=24, num_attention_heads=16,
+                          intermediate_size=4096, hidden_dropout_prob=0.0, attention_probs_dropout_prob=0.0,
+                          max_position_embeddings=512, type_vocab_size=0, relative_attention=True, position_buckets=256,
+                          max_relative_positions=512, share_att_key=True, pos_att_type=["c2p", "p2c"],
+                          norm_rel_ebd="layer_norm", position_biased_input=False, layer_norm_eps=1e-7,
+                          initializer_range=0.02)
+    torch.manual_seed(0)
+    with torch.device("cuda:0"):
+        truth = DebertaV2Model(cfg).eval()                                    # float32 eager: the yardstick
+    import copy
+    theirs = copy.deepcopy(truth).to(torch.bfloat16)
+    ours = patch_model(copy.deepcopy(truth).to(torch.bfloat16))
+    rs = np.random.RandomState(0)
+    lens = rs.randint(64, 513, size=16)
+    ids = torch.from_numpy(rs.randint(0, 128000, size=(16, 512))).cuda()
+    mask = torch.from_numpy((np.arange(512)[None] < lens[:, None]).astype(np.int64)).cuda()
+    valid = mask.bool()
+    print("[case] config 4: v3-large-shaped encoder, b16 x L512, bf16", flush=True)
+    with torch.no_grad():
+        t = truth(input_ids=ids, attention_mask=mask).last_hidden_state
+        b = theirs(input_ids=ids, attention_mask=mask).last_hidden_state.float()
+        packed = ours(input_ids=ids, attention_mask=mask).last_hidden_state.float()
+        ours.encoder.pack_sequences = False
+        padded = ours(input_ids=ids, attention_mask=mask).last_hidden_state.float()
+    assert packed[~valid].abs().max().item() == 0.0
+    err_hf = (b[valid] - t[valid]).abs()
+    for name, a in (("packed", packed), ("padded", padded)):
+        assert torch.isfinite(a).all(), name
+        err = (a[valid] - t[valid]).abs()
+        print(f"  {name}: mean |err| {err.mean().item():.4e} (HF bf16 eager {err_hf.mean().item():.4e}), "
+              f"max {err.max().item():.4e} (HF {err_hf.max().item():.4e})", flush=True)
+        assert err.mean().item() <= 1.25 * err_hf.mean().item() + 1e-4, name
+        assert err.max().item() <= 1.5 * err_hf.max().item() + 1e-3, name
+    assert (packed[valid] - padded[valid]).abs().max().item() <= 1.5 * err_hf.max().item() + 1e-3

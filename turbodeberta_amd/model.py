@@ -50,7 +50,7 @@ from transformers.models.deberta_v2.modeling_deberta_v2 import (
 
 from .ops.flash_attention import flash_attention_with_disentangled
 from .ops.flash_attention_varlen import flash_attention_with_disentangled_varlen
-from .padding import _get_unpad_data, index_first_axis, key_padding_mask, pad_input
+from .padding import index_first_axis, key_padding_mask, pad_input
 
 
 def _versions(*tensors):
@@ -59,19 +59,63 @@ def _versions(*tensors):
     return tuple((id(t), t.data_ptr(), t._version, t.dtype, t.device) if t is not None else None for t in tensors)
 
 
-def _lengths_of(attention_mask):
-    """int32 [B] valid lengths of a right-padded batch.  The result is attached to the mask tensor, so the
-    layers of an encoder, which all receive the same mask object (modeling_deberta_v2.py:651-660), compute it
-    once per forward."""
-    cached = getattr(attention_mask, "_tdb_lengths", None)
-    if cached is not None and cached[0] == attention_mask._version:
-        return cached[1]
-    lengths = key_padding_mask(attention_mask).sum(dim=-1, dtype=torch.int32)
+def _version_of(t):
+    """In-place modification counter of a tensor, or None where there is none to read (inference tensors do not
+    track one and raise on access)."""
     try:
-        attention_mask._tdb_lengths = (attention_mask._version, lengths)
+        return t._version
+    except (RuntimeError, AttributeError):
+        return None
+
+
+class _MaskInfo:
+    """What the fused paths need to know about an attention mask: ``lengths`` int32 ``[B]`` on the device and
+    ``total``, the number of valid tokens (a host int)."""
+    __slots__ = ("lengths", "total")
+
+    def __init__(self, lengths, total):
+        self.lengths, self.total = lengths, total
+
+
+def _mask_info(attention_mask):
+    """Valid lengths of a batch whose mask is **right padded** (valid tokens first), verified: the kernels take
+    per-sequence lengths, so a mask with holes or left padding cannot be expressed and raises ``ValueError`` instead
+    of attending to the wrong tokens.  A 3-D / 4-D mask must be the outer product ``m_i * m_j`` Hugging Face's
+    encoder builds (modeling_deberta_v2.py:601-608).  The check costs one host synchronisation per mask object;
+    the result is attached to the tensor, so the layers of an encoder, which all receive the same mask object
+    (modeling_deberta_v2.py:651-660), share it.  (A mask without a modification counter -- an inference tensor --
+    is trusted not to be modified in place between calls.)"""
+    version = _version_of(attention_mask)
+    cached = getattr(attention_mask, "_tdb_info", None)
+    if cached is not None and cached[0] == version:
+        return cached[1]
+    valid = key_padding_mask(attention_mask) != 0                               # [B, L]
+    L = valid.shape[-1]
+    lengths = valid.sum(dim=-1, dtype=torch.int32)
+    ok = (valid == (torch.arange(L, device=valid.device)[None, :] < lengths[:, None])).all()
+    if attention_mask.dim() > 2:
+        full = attention_mask if attention_mask.dim() == 3 else attention_mask[:, 0]
+        ok = ok & ((full != 0) == (valid[:, :, None] & valid[:, None, :])).all()
+    ok_host, total = torch.stack([ok.to(torch.int64), lengths.sum(dtype=torch.int64)]).tolist()   # the one synchronisation
+    if not ok_host:
+        raise ValueError("attention_mask must be right padded (valid tokens first, no holes) and, if 3-D or 4-D, the "
+                         "outer product of a key-padding mask with itself: the fused attention takes per-sequence "
+                         "lengths.  Use the eager Hugging Face modules for other masks.")
+    info = _MaskInfo(lengths, int(total))
+    try:
+        attention_mask._tdb_info = (version, info)
     except AttributeError:      # tensor subclasses without a __dict__
         pass
-    return lengths
+    return info
+
+
+def _packing_of(info, batch, seqlen, device):
+    """``(indices, cu_seqlens)`` of a verified right-padded batch without a further synchronisation: positions of the
+    valid tokens in the flattened ``[B*L]`` batch, int32 boundaries with a leading 0."""
+    cu = torch.nn.functional.pad(torch.cumsum(info.lengths, dim=0, dtype=torch.int32), (1, 0))
+    seq = torch.repeat_interleave(torch.arange(batch, device=device), info.lengths.long(), output_size=info.total)
+    indices = torch.arange(info.total, device=device) - cu[:-1].long()[seq] + seq * seqlen
+    return indices, cu
 
 
 class FlashDisentangledSelfAttention(DisentangledSelfAttention):
@@ -79,7 +123,9 @@ class FlashDisentangledSelfAttention(DisentangledSelfAttention):
     product replaced by one kernel launch.  Same constructor, parameters and ``forward`` signature.
 
     Masks: sequences must be right-padded (valid tokens first), which is what the DeBERTa tokenizers
-    produce; the valid length of each sequence is taken from the mask.  Rows of padded query tokens
+    produce; the valid length of each sequence is taken from the mask, and a mask of any other shape
+    (holes, left padding, a 3-D / 4-D mask that is not ``m_i * m_j``) raises ``ValueError`` -- checked
+    once per mask object, with one host synchronisation.  Rows of padded query tokens
     are returned as zeros (the eager module gives them a meaningless uniform average,
     modeling_deberta_v2.py:256-259); downstream layers mask them anyway.
     ``output_attentions=True`` needs the probability matrix, which the fused kernel never forms: that
@@ -111,7 +157,7 @@ class FlashDisentangledSelfAttention(DisentangledSelfAttention):
 
         pos_key, pos_query, sm_scale, buckets, max_rel = self._position_terms(rel_embeddings, hidden_states.dtype,
                                                                               frozen)
-        seqlens = _lengths_of(attention_mask) if attention_mask is not None else None
+        seqlens = _mask_info(attention_mask).lengths if attention_mask is not None else None
         out = flash_attention_with_disentangled(q, k, v, None, None, False, sm_scale, buckets, max_rel,
                                                 pos_key_layer=pos_key, pos_query_layer=pos_query,
                                                 seqlens_k=seqlens)
@@ -129,7 +175,8 @@ class FlashDisentangledSelfAttention(DisentangledSelfAttention):
         pos_key, pos_query, sm_scale, buckets, max_rel = self._position_terms(rel_embeddings, hidden_states.dtype, True)
         out = flash_attention_with_disentangled_varlen(qkv[:, 0], qkv[:, 1], qkv[:, 2], None, None, cu_seqlens,
                                                        cu_seqlens, max_seqlen, max_seqlen, False, sm_scale, buckets,
-                                                       max_rel, pos_key_layer=pos_key, pos_query_layer=pos_query)
+                                                       max_rel, pos_key_layer=pos_key, pos_query_layer=pos_query,
+                                                       zero_output=False)      # the packing comes from the verified mask
         return out.reshape(T, H * D)
 
     def _position_terms(self, rel_embeddings, dtype, frozen):
@@ -212,10 +259,11 @@ class FlashDebertaV2Encoder(DebertaV2Encoder):
     In eval mode under ``torch.no_grad()`` a batch that contains padding runs **packed**: the valid tokens
     are gathered once, every layer works on ``[valid_tokens, hidden]`` (``forward_packed`` of the attention
     module, then Hugging Face's own output / feed-forward submodules, which are shape agnostic), and the
-    result is scattered back to ``[B, L, hidden]`` with zeros at padded positions.  Counting the valid
-    tokens is the only host synchronisation of the forward.  Everything else -- training, gradients,
-    ``output_attentions``, ``query_states``, masks that are not ``[B, L]``-reducible, CPU tensors, batches
-    without padding -- takes the parent's loop over the (fused, padded) layers.
+    result is scattered back to ``[B, L, hidden]`` with zeros at padded positions.  Verifying the mask and
+    counting the valid tokens is the only host synchronisation of the forward.  Everything else -- training,
+    gradients, ``output_attentions``, ``query_states``, CPU tensors, batches without padding -- takes the
+    parent's loop over the (fused, padded) layers.  Masks must be right padded in either path (see
+    ``FlashDisentangledSelfAttention``); others raise ``ValueError``.
 
     ``pack_sequences = False`` switches the packed path off."""
 
@@ -254,8 +302,10 @@ class FlashDebertaV2Encoder(DebertaV2Encoder):
                     and query_states is None and hidden_states.is_cuda and attention_mask.dim() in (2, 3, 4))
         if packable:
             B, L, _ = hidden_states.shape
-            indices, cu_seqlens, _ = _get_unpad_data(attention_mask)       # the one host synchronisation
-            packable = indices.numel() < B * L
+            info = _mask_info(attention_mask)                                # the one host synchronisation
+            packable = info.total < B * L
+            if packable:
+                indices, cu_seqlens = _packing_of(info, B, L, hidden_states.device)
         if not packable:
             if fused and relative_pos is None and self.relative_attention:
                 relative_pos = hidden_states.new_empty(0)    # fused layers never read the [L, L] matrix: do not build it

@@ -18,8 +18,15 @@ from . import _launch as L
 
 def prepare(q, k, v, q_pos, k_pos, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, causal=False, sm_scale=None,
             position_buckets=0, max_relative_distance=0, *, pos_key_layer=None, pos_query_layer=None,
-            force_generic=False) -> L.PreparedLaunch:
-    """Validate and pack one call of ``flash_attention_with_disentangled_varlen`` without launching it."""
+            force_generic=False, check_cu_seqlens=False, zero_output=True) -> L.PreparedLaunch:
+    """Validate and pack one call of ``flash_attention_with_disentangled_varlen`` without launching it.
+
+    ``max_seqlen`` must be a true upper bound and ``cu_seqlens[-1]`` must equal the token count: the kernels
+    clamp a longer sequence to ``max_seqlen`` and never touch rows past ``cu_seqlens[-1]``.  Neither can be
+    seen without reading ``cu_seqlens`` on the host, so the default makes no such read; rows the kernels do
+    not cover are zeros (``zero_output``; callers that know their packing is exact, like the packed encoder,
+    pass False and save the fill).  ``check_cu_seqlens=True`` copies the offsets to the host (one
+    synchronisation) and raises ``ValueError`` on the first inconsistency."""
     if q.dim() != 3 or k.dim() != 3 or v.dim() != 3:
         raise ValueError("q, k, v must be [total_tokens, H, D]")
     Dq, Dk, Dv = q.shape[-1], k.shape[-1], v.shape[-1]
@@ -44,10 +51,13 @@ def prepare(q, k, v, q_pos, k_pos, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max
     B = cu_seqlens_q.numel() - 1
     span = L.att_span(position_buckets, max_relative_distance)
     q, k, v = L.as_rows(q), L.as_rows(k), L.as_rows(v)
-    o = torch.empty_like(q)
+    make = torch.zeros if zero_output else torch.empty
+    o = (torch.zeros_like if zero_output else torch.empty_like)(q)
     if not L.rows_ok(o):
-        o = torch.empty(q.shape, dtype=q.dtype, device=dev)
+        o = make(q.shape, dtype=q.dtype, device=dev)
     cu = cu_seqlens_q.to(torch.int32).contiguous()
+    if check_cu_seqlens:
+        _lib.check_cu_seqlens(cu.cpu().numpy(), T, max(int(max_seqlen_q), 1))
     keep = [cu, q, k, v]
 
     a = _lib.VarlenArgs()
@@ -87,10 +97,12 @@ class FlashAttentionDisentangled(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, q, k, v, q_pos, k_pos, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, causal,
-                sm_scale, position_buckets, max_relative_distance, pos_key_layer, pos_query_layer, force_generic):
+                sm_scale, position_buckets, max_relative_distance, pos_key_layer, pos_query_layer, force_generic,
+                check_cu_seqlens=False, zero_output=True):
         return prepare(q, k, v, q_pos, k_pos, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, causal,
                        sm_scale, position_buckets, max_relative_distance, pos_key_layer=pos_key_layer,
-                       pos_query_layer=pos_query_layer, force_generic=force_generic).launch()
+                       pos_query_layer=pos_query_layer, force_generic=force_generic,
+                       check_cu_seqlens=check_cu_seqlens, zero_output=zero_output).launch()
 
     @staticmethod
     def backward(ctx, grad_output):
@@ -102,7 +114,8 @@ def flash_attention_with_disentangled_varlen(q, k, v, q_pos, k_pos, cu_seqlens_q
                                              position_buckets=0, max_relative_distance=0, *,
                                              pos_key_layer: Optional[torch.Tensor] = None,
                                              pos_query_layer: Optional[torch.Tensor] = None,
-                                             force_generic: bool = False):
+                                             force_generic: bool = False, check_cu_seqlens: bool = False,
+                                             zero_output: bool = True):
     """Packed-sequence form of ``flash_attention_with_disentangled``.
 
     Positional parameters are the reference's (ops/flash_attention_varlen.py:348-374):
@@ -111,13 +124,17 @@ def flash_attention_with_disentangled_varlen(q, k, v, q_pos, k_pos, cu_seqlens_q
     q_pos, k_pos : c2p / p2c strips ``[total_tokens, H, 2*span]`` or None.
     cu_seqlens_q, cu_seqlens_k : int32 ``[B+1]`` cumulative lengths (leading 0), as produced by
         ``padding._get_unpad_data``; both must describe the same packing.
-    max_seqlen_q, max_seqlen_k : longest sequence (an upper bound is fine).
+    max_seqlen_q, max_seqlen_k : longest sequence (an upper bound is fine; a smaller value truncates longer
+        sequences, their remaining rows come back as zeros).
     causal, sm_scale, position_buckets, max_relative_distance : as in the fixed-length operator.
 
     Keyword-only: ``pos_key_layer`` / ``pos_query_layer`` ``[H, 2*span, D]`` fused tables,
-    ``force_generic``.  Relative positions are in-sequence offsets
+    ``force_generic``, ``check_cu_seqlens`` (validate the offsets on the host: one synchronisation,
+    ``ValueError`` when they are malformed, exceed ``max_seqlen`` or do not end at the token count) and
+    ``zero_output`` (see ``prepare``).  Relative positions are in-sequence offsets
     (ops/flash_attention_varlen.py:70,118); each key is masked by its own sequence's length.
-    No host synchronisation is made.  Returns ``o [total_tokens, H, D]``; forward only."""
+    No host synchronisation is made unless ``check_cu_seqlens`` asks for one.  Returns ``o [total_tokens, H, D]``; forward only."""
     return FlashAttentionDisentangled.apply(q, k, v, q_pos, k_pos, cu_seqlens_q, cu_seqlens_k, max_seqlen_q,
                                             max_seqlen_k, causal, sm_scale, position_buckets,
-                                            max_relative_distance, pos_key_layer, pos_query_layer, force_generic)
+                                            max_relative_distance, pos_key_layer, pos_query_layer, force_generic,
+                                            check_cu_seqlens, zero_output)
