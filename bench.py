@@ -6,13 +6,21 @@ A "step" is one attention forward over one batch of synthetic DeBERTa-v3-base at
 
   fixed   batch 32 x seq 512, right-padded, valid lengths uniform in [384, 512]   (headline `value`)
   varlen  64 sequences with lengths uniform in [16, 512], packed with cu_seqlens  (reported beside it)
+  long    batch 4 x seq 4096, full mask, and its packed variant (8 sequences U[1024, 4096])   (`long`, `long_varlen`)
+  generic the vector-ALU kernel that serves float32 inputs and the strip-taking signature: the attention of the
+          config-1 layer (batch 2 x seq 128, float32) and a strip-mode call at batch 8 x seq 256 in bf16   (`generic`)
 
 Prints ONE JSON line.  `value` is algorithmic attention TFLOP/s of the fixed workload over the timed
 region; FLOPs per sequence of valid length l and per head:  4*l*l*d (QK^T + PV) + 4*l*W*d (c2p + p2c),
 W = min(2*span, 2*l - 1) -- no credit for padding, window recompute or projections.
 `roofline` prices the kernel's average launch duration (two HIP events on the launch stream that bracket the timed
 region, divided by the number of launches) against the MI355X dense bf16 MFMA peak; `cpu_baseline` times the CPU oracle (eager float32 restatement of
-Hugging Face's DisentangledSelfAttention) on a bounded sample of the same workload.
+Hugging Face's DisentangledSelfAttention) on a bounded sample of the same workload and on the config-1 layer.
+
+Before the warm-up launches of every workload the GPU is kept busy for `--prewarm-ms` (default 30 ms of launches of
+that workload, untimed, reported as `prewarm_ms`): the first milliseconds of load after an idle period run at a lower
+clock, and the timed region of a short run (`--steps 20 --warmup 5` is 2.5 ms) would otherwise sit inside that ramp.
+`--warmup` and `--steps` keep their meaning.
 """
 from __future__ import annotations
 
@@ -34,19 +42,43 @@ BUCKETS, MAX_REL, SPAN = 256, 512, 256
 PEAK_BF16_TFLOPS = 2500.0       # MI355X dense bf16 MFMA, AMD public spec
 PEAK_HBM_GBS = 8000.0
 METRIC = "attn TFLOP/s + tokens/s, DeBERTa-v3-base b32xL512 bf16, fixed and varlen"
-# HBM bytes per launch from `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` runs of this script, each counter scaled
-# by what it reads for a plain 512 MiB device copy (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000); the runs and raw counter
-# values are recorded in profiles/attn_mfma_kernel_fixed_b32xL512.md and profiles/attn_mfma_kernel_varlen_64seq.md.
-MEASURED_TRAFFIC_BYTES = {"fixed": 104.1e6, "varlen": 210.3e6}
+PEAK_FP32_VALU_TFLOPS = 157.3   # MI355X vector fp32, AMD public spec (what the generic kernel is priced against)
+# HBM bytes per launch are not measured by this script: they come from `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE`
+# runs of it, each counter scaled by what it reads for a plain 512 MiB device copy.  The figures, the commands and the
+# commit they were taken at are recorded in the files named here; `roofline.traffic` repeats them with that source.
+RECORDED_TRAFFIC = {
+    "fixed": ("profiles/attn_mfma_kernel_fixed_b32xL512.md", None),
+    "varlen": ("profiles/attn_mfma_kernel_varlen_64seq.md", None),
+}
 
 
-def flops_of(lengths) -> float:
+def recorded_traffic(name):
+    """(bytes, source) from the profile summary of a workload: the line `traffic_bytes_per_launch: <number>` and the
+    line `commit: <hash>` of the file; (None, None) when the file or the line is missing."""
+    path = RECORDED_TRAFFIC.get(name, (None, None))[0]
+    if path is None:
+        return None, None
+    try:
+        text = open(os.path.join(ROOT, path)).read()
+    except OSError:
+        return None, None
+    val = commit = None
+    for line in text.splitlines():
+        if line.startswith("traffic_bytes_per_launch:"):
+            val = float(line.split(":", 1)[1])
+        if line.startswith("commit:"):
+            commit = line.split(":", 1)[1].strip()
+    return val, (f"{path} (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, calibrated on a 512 MiB copy; commit {commit})"
+                 if val is not None else None)
+
+
+def flops_of(lengths, heads=H) -> float:
     tot = 0.0
     for l in lengths:
         l = int(l)
         w = min(2 * SPAN, 2 * l - 1)
         tot += 4.0 * l * l * D + 4.0 * l * w * D
-    return H * tot
+    return heads * tot
 
 
 def algorithmic_bytes(lengths) -> float:
@@ -84,10 +116,48 @@ def build_fixed(dev, B=32, L=512):
     return plan, lengths, dict(q=q, k=k, v=v, pk=pk, pq=pq)
 
 
-def build_varlen(dev, n_seq=64):
+def build_long(dev, B=4, L=4096):
+    """Config 5: batch 4 x seq 4096, full mask."""
+    from turbodeberta_amd.ops import flash_attention as fa
+    w, g = make_weights(dev)
+    hidden = torch.randn(B, L, HID, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    lin = torch.nn.functional.linear
+    heads = lambda x: x.view(B, L, H, D).permute(0, 2, 1, 3)
+    q, k, v = heads(lin(hidden, w["wq"])), heads(lin(hidden, w["wk"])), heads(lin(hidden, w["wv"]))
+    pk, pq = position_tables(w)
+    plan = fa.prepare(q, k, v, None, None, False, 1.0 / math.sqrt(3 * D), BUCKETS, MAX_REL,
+                      pos_key_layer=pk, pos_query_layer=pq)
+    return plan, np.full(B, L)
+
+
+def build_generic(dev):
+    """The two callers of the vector-ALU kernel: (a) the attention of the config-1 layer -- batch 2 x seq 128, 12 heads,
+    float32, full mask; (b) the reference's literal call shape -- c2p / p2c strips [B, H, L, 2*span] computed by the
+    caller (model.py:122-137 of the reference) -- at batch 8 x seq 256 in bf16."""
+    from turbodeberta_amd.ops import flash_attention as fa
+    w, g = make_weights(dev)
+    lin = torch.nn.functional.linear
+    out = {}
+    for name, (B, L, dt) in {"config1_fp32": (2, 128, torch.float32), "strips_bf16": (8, 256, torch.bfloat16)}.items():
+        hidden = torch.randn(B, L, HID, generator=g, device=dev, dtype=torch.float32).to(dt)
+        heads = lambda x: x.view(B, L, H, D).permute(0, 2, 1, 3)
+        q, k, v = (heads(lin(hidden, w[n].to(dt))) for n in ("wq", "wk", "wv"))
+        pk, pq = (t.to(dt) for t in position_tables(w))
+        if name == "strips_bf16":
+            c2p = torch.matmul(q, pk.transpose(-1, -2)[None])
+            p2c = torch.matmul(k, pq.transpose(-1, -2)[None])
+            plan = fa.prepare(q, k, v, c2p, p2c, False, 1.0 / math.sqrt(3 * D), BUCKETS, MAX_REL)
+        else:
+            plan = fa.prepare(q, k, v, None, None, False, 1.0 / math.sqrt(3 * D), BUCKETS, MAX_REL,
+                              pos_key_layer=pk, pos_query_layer=pq)
+        out[name] = (plan, np.full(B, L))
+    return out
+
+
+def build_varlen(dev, n_seq=64, lo=16, hi=512):
     from turbodeberta_amd.ops import flash_attention_varlen as fv
     w, g = make_weights(dev)
-    lengths = np.random.RandomState(0).randint(16, 513, size=n_seq)
+    lengths = np.random.RandomState(0).randint(lo, hi + 1, size=n_seq)
     T = int(lengths.sum())
     hidden = torch.randn(T, HID, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
     lin = torch.nn.functional.linear
@@ -99,11 +169,29 @@ def build_varlen(dev, n_seq=64):
     return plan, lengths
 
 
-def time_steps(plan, steps, warmup):
-    """Times exactly `steps` back-to-back launches after `warmup` untimed ones.  Returns
+def prewarm(plan, budget_ms):
+    """Keeps the GPU busy with launches of `plan` until `budget_ms` of wall clock have passed; returns the ms spent."""
+    if budget_ms <= 0:
+        return 0.0
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    while True:
+        for _ in range(20):
+            plan.launch()
+        torch.cuda.synchronize()
+        spent = (time.perf_counter() - t0) * 1e3
+        if spent >= budget_ms:
+            return spent
+
+
+def time_steps(plan, steps, warmup, prewarm_ms=0.0):
+    """Times exactly `steps` back-to-back launches after `warmup` untimed ones (and, before those, `prewarm_ms` of
+    untimed launches that bring the clock up).  Returns
     (wall ms per step between two synchronisations, kernel ms = span between two HIP events that bracket the same
     timed region on the launch stream / steps, then median and minimum of per-launch event pairs from a second pass;
-    an event pair around a single launch reads about 3 us more than the launch takes in a back-to-back stream)."""
+    an event pair around a single launch reads about 3 us more than the launch takes in a back-to-back stream;
+    ms spent pre-warming)."""
+    spent = prewarm(plan, prewarm_ms)
     for _ in range(warmup):
         plan.launch()
     torch.cuda.synchronize()
@@ -123,7 +211,7 @@ def time_steps(plan, steps, warmup):
         b.record()
     torch.cuda.synchronize()
     durs = sorted(a.elapsed_time(b) for a, b in ev)
-    return wall_ms, span_ms, durs[len(durs) // 2], durs[0]
+    return wall_ms, span_ms, durs[len(durs) // 2], durs[0], spent
 
 
 def cpu_baseline(tensors, lengths, budget_s=12.0):
@@ -147,7 +235,38 @@ def cpu_baseline(tensors, lengths, budget_s=12.0):
     return {"value": round(flops_of(lengths[:nb]) / med / 1e12, 5), "unit": "TFLOP/s", "cores": torch.get_num_threads(),
             "kind": "port", "ms_per_sample": round(med * 1e3, 2),
             "sample": f"first {nb} of the 32 sequences of the fixed workload (lengths {lengths[:nb].tolist()}), "
-                      f"float32 torch-CPU oracle, median of {len(times)} runs"}
+                      f"float32 torch-CPU oracle, median of {len(times)} runs",
+            "config1_layer": cpu_config1_layer()}
+
+
+def cpu_config1_layer(budget_s=6.0):
+    """BASELINE config 1 on the host: one DisentangledSelfAttention layer from hidden states (projections, position
+    tables, attention), batch 2 x seq 128 x hidden 768, 12 heads, float32, full mask, seed 0 -- the oracle's
+    restatement of the eager layer."""
+    from oracle import hf_eager as O
+    g = torch.Generator().manual_seed(0)
+    B, L = 2, 128
+    hidden = torch.randn(B, L, HID, generator=g)
+    rel = torch.randn(2 * SPAN, HID, generator=g)
+    wq, wk, wv = (torch.randn(HID, HID, generator=g) * 0.02 for _ in range(3))
+    zero = torch.zeros(HID)
+    mask = O.encoder_attention_mask(torch.ones(B, L, dtype=torch.long))
+    run = lambda: O.self_attention_layer(hidden, mask, rel, wq, zero, wk, zero, wv, zero, H, position_buckets=BUCKETS,
+                                         max_relative_positions=MAX_REL)
+    run()
+    run()
+    times, t_start = [], time.perf_counter()
+    while len(times) < 5 or (time.perf_counter() - t_start < budget_s and len(times) < 200):
+        t0 = time.perf_counter()
+        run()
+        times.append(time.perf_counter() - t0)
+    med = float(np.median(times))
+    attn_flops = flops_of([L] * B)
+    proj_flops = 2.0 * HID * HID * (3 * B * L + 2 * 2 * SPAN)
+    return {"ms_per_layer": round(med * 1e3, 3), "tokens_per_s": round(B * L / med, 1),
+            "attention_gflops": round(attn_flops / med / 1e9, 2), "with_projections_gflops": round((attn_flops + proj_flops) / med / 1e9, 2),
+            "cores": torch.get_num_threads(),
+            "sample": f"whole layer, batch {B} x seq {L} x hidden {HID}, float32, median of {len(times)} runs"}
 
 
 def model_benchmark(dev, steps=30, warmup=10):
@@ -204,11 +323,13 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=200,
-                    help="untimed launches before the timed region (the first ~2 ms of load after an idle period run "
-                         "at a lower clock: 200 launches = 20 ms get past that)")
+    ap.add_argument("--warmup", type=int, default=20, help="untimed launches right before the timed region")
+    ap.add_argument("--prewarm-ms", type=float, default=30.0,
+                    help="untimed launches of the workload for this many ms before the warm-up, to get past the clock "
+                         "ramp that follows an idle period (0 switches it off)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--workload", choices=["both", "fixed", "varlen"], default="both")
+    ap.add_argument("--workload", choices=["all", "both", "fixed", "varlen", "long", "generic"], default="all",
+                    help="all = fixed + varlen + long + long_varlen + generic; both = fixed + varlen")
     ap.add_argument("--with-model", action="store_true",
                     help="add the end-to-end forward of a v3-large-shaped model (fused attention vs Hugging Face eager "
                          "attention on the same GPU) to the JSON line as \"model\"")
@@ -235,17 +356,21 @@ def main():
 
     out = {"metric": METRIC, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic"}
+    spent_prewarm = []
 
-    def measure(plan, lengths, name, kernel):
-        wall_ms, mean_ms, med_ms, min_ms = time_steps(plan, args.steps, args.warmup)
+    def measure(plan, lengths, name, kernel, peak=PEAK_BF16_TFLOPS, bound="mfma", steps=None):
+        steps = steps or args.steps
+        wall_ms, mean_ms, med_ms, min_ms, spent = time_steps(plan, steps, args.warmup, args.prewarm_ms)
+        spent_prewarm.append(spent)
         fl = flops_of(lengths)
         ach = fl / (mean_ms * 1e-3) / 1e12
+        traffic, traffic_source = recorded_traffic(name)
         return {
-            "value": round(fl / (wall_ms * 1e-3) / 1e12, 2), "ms_per_step": round(wall_ms, 4),
+            "value": round(fl / (wall_ms * 1e-3) / 1e12, 2), "ms_per_step": round(wall_ms, 4), "steps": steps,
             "tokens_per_s": round(float(lengths.sum()) / (wall_ms * 1e-3), 1),
             "core_tflops": round(H * sum(4.0 * int(l) ** 2 * D for l in lengths) / (wall_ms * 1e-3) / 1e12, 2),
-            "roofline": {"bound": "mfma", "achieved": round(ach, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                         "frac": round(ach / PEAK_BF16_TFLOPS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(name), "kernel": kernel,
+            "roofline": {"bound": bound, "achieved": round(ach, 2), "peak": peak, "unit": "TFLOP/s",
+                         "frac": round(ach / peak, 4), "traffic": traffic, "traffic_source": traffic_source, "kernel": kernel,
                          "kernel_ms_mean": round(mean_ms, 4), "kernel_ms_pair_median": round(med_ms, 4),
                          "kernel_ms_pair_min": round(min_ms, 4), "algorithmic_gflop": round(fl / 1e9, 3), "algorithmic_bytes": algorithmic_bytes(lengths),
                          "hbm_gbs_algorithmic": round(algorithmic_bytes(lengths) / (mean_ms * 1e-3) / 1e9, 1)},
@@ -253,13 +378,30 @@ def main():
 
     res_fixed = res_var = None
     tensors = lengths_f = None
-    if args.workload in ("both", "fixed"):
+    if args.workload in ("all", "both", "fixed"):
         plan, lengths_f, tensors = build_fixed(dev)
         res_fixed = measure(plan, lengths_f, "fixed", "attn_mfma_kernel<c2p,p2c>")
-    if args.workload in ("both", "varlen"):
+    if args.workload in ("all", "both", "varlen"):
         plan_v, lengths_v = build_varlen(dev)
         res_var = measure(plan_v, lengths_v, "varlen", "attn_mfma_kernel<c2p,p2c>")
-    head = res_fixed or res_var
+    extra = {}
+    if args.workload in ("all", "long"):
+        few = max(5, min(args.steps, 40))                      # a launch takes ~1 ms: fewer steps keep the run short
+        plan_l, lengths_l = build_long(dev)
+        extra["long"] = {"workload": "fixed b4xL4096, full mask, 12 heads x 64, buckets 256, max_rel 512, c2p|p2c",
+                         **measure(plan_l, lengths_l, "long", "attn_mfma_kernel<c2p,p2c>", steps=few)}
+        del plan_l
+        plan_lv, lengths_lv = build_varlen(dev, n_seq=8, lo=1024, hi=4096)
+        extra["long_varlen"] = {"workload": "8 packed sequences, lengths U[1024,4096] seed 0, total tokens %d" % int(lengths_lv.sum()),
+                                **measure(plan_lv, lengths_lv, "long_varlen", "attn_mfma_kernel<c2p,p2c>", steps=few)}
+        del plan_lv
+    if args.workload in ("all", "generic"):
+        notes = {"config1_fp32": "attention of the config-1 layer: batch 2 x seq 128, 12 heads x 64, float32, fused tables",
+                 "strips_bf16": "strip-taking signature (c2p / p2c strips [B,H,L,512] from the caller), batch 8 x seq 256, bf16"}
+        extra["generic"] = {name: {"workload": notes[name],
+                                   **measure(pl, ln, name, "attn_generic_kernel", peak=PEAK_FP32_VALU_TFLOPS, bound="valu")}
+                            for name, (pl, ln) in build_generic(dev).items()}
+    head = res_fixed or res_var or extra.get("long") or next(iter(extra["generic"].values()))
     out.update({"value": head["value"], "ms_per_step": head["ms_per_step"], "tokens_per_s": head["tokens_per_s"],
                 "core_tflops": head["core_tflops"], "roofline": head["roofline"]})
     out["config"] = {"workload": ("fixed b32xL512, valid lengths U[384,512] seed 0" if res_fixed else
@@ -268,6 +410,8 @@ def main():
     if res_fixed and res_var:
         out["varlen"] = {"workload": "64 packed sequences, lengths U[16,512] seed 0, total tokens %d" % int(lengths_v.sum()),
                          **res_var}
+    out.update(extra)
+    out["prewarm_ms"] = round(float(np.mean(spent_prewarm)), 2) if spent_prewarm else 0.0
     if not args.no_cpu_baseline and tensors is not None:
         out["cpu_baseline"] = cpu_baseline(tensors, lengths_f)
     if args.with_model:
