@@ -86,7 +86,11 @@ struct Elem<TDB_BF16> {
     using X2 = bf16x2;
     using X8 = bf16x8;
     static __device__ __forceinline__ f32x16 mfma(X8 a, X8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
-    static __device__ __forceinline__ float widen(uint16_t raw) { return __builtin_bit_cast(float, uint32_t(raw) << 16); }
+    // One half of a dword as fp32 through a byte permute (the selector says which half): bf16 -> fp32 is a shift.
+    static constexpr uint32_t PICK_LO = 0x05040c0cu, PICK_HI = 0x07060c0cu;
+    static __device__ __forceinline__ float pick(uint32_t pair, uint32_t sel) {
+        return __builtin_bit_cast(float, __builtin_amdgcn_perm(pair, 0u, sel));
+    }
 };
 template <>
 struct Elem<TDB_F16> {
@@ -94,7 +98,10 @@ struct Elem<TDB_F16> {
     using X2 = f16x2;
     using X8 = f16x8;
     static __device__ __forceinline__ f32x16 mfma(X8 a, X8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
-    static __device__ __forceinline__ float widen(uint16_t raw) { return (float)__builtin_bit_cast(_Float16, raw); }
+    static constexpr uint32_t PICK_LO = 0x0c0c0504u, PICK_HI = 0x0c0c0706u;
+    static __device__ __forceinline__ float pick(uint32_t pair, uint32_t sel) {
+        return (float)__builtin_bit_cast(X2, __builtin_amdgcn_perm(pair, 0u, sel))[0];
+    }
 };
 
 template <typename X8>
@@ -785,7 +792,6 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         //      position terms of step s: c2p as four B operands of 16 keys each, straight out of the ring (keys
         //      64s .. 64s+63 never straddle its wrap), p2c element by element: (key jj, query n) takes
         //      P'[jj][w + 4n + 63 - jj], converted to fp32 into what becomes the initial score accumulator ----------
-        store_kv(s & 1, s + 2 < nsteps);  // (in the last step the key buffers already take the next tile's keys)
         X8 cf[2][2];
         if (HAS_C2P) {
 #pragma unroll
@@ -795,13 +801,30 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         }
         f32x16 s_acc[2];
         if (HAS_P2C) {
-            // The gathers are ordinary LDS loads; the compiler places the waits.  (Loads issued from inline assembly
-            // would be invisible to it: it may then copy a destination register before the data has arrived.)
-            const auto* pbase = TDB_LDS(const uint16_t, sm.p) + (w + 63 + 4 * il) + 4 * hh * (PS - 1);
+            // Element (key jc, query n) sits at 16-bit index X + jc * (PS - 1), X = w + 63 + 4n: from one key to the next
+            // the index moves by an odd amount, so the element alternates between the low and the high half of its
+            // dword with the parity of jc, starting from the parity of w + 1 -- the same for every lane, because the
+            // rows of a wave are 4 apart.  The dwords of keys jc and jc + 2 are (PS - 1) dwords apart: one two-address
+            // read fetches both; a byte permute with a wave-uniform selector moves the wanted half into an fp32.
+            // The gathers are ordinary LDS loads; the compiler pairs them and places the waits.  (Loads issued from
+            // inline assembly would be invisible to it: it may then copy a destination register before the data has arrived.)
+            constexpr int PD = PS - 1;            // dwords between the elements of keys jc and jc + 2
+            const int px = (w + 1) & 1;
+            const auto* p_even = TDB_LDS(const uint32_t, sm.p) + ((w + 63 + 4 * il) >> 1) + 2 * hh * PD;    // key 4hh
+            const auto* p_odd = p_even + PD / 2 + px;                                                          // key 4hh + 1
+            const uint32_t sel_even = px ? E::PICK_HI : E::PICK_LO, sel_odd = px ? E::PICK_LO : E::PICK_HI;
+            uint32_t g[2][16];
 #pragma unroll
             for (int jt = 0; jt < 2; ++jt)
 #pragma unroll
-                for (int e = 0; e < 16; ++e) s_acc[jt][e] = E::widen(pbase[(32 * jt + 8 * (e >> 2) + (e & 3)) * (PS - 1)]);
+                for (int e = 0; e < 16; ++e) {
+                    const int jc = 32 * jt + 8 * (e >> 2) + (e & 3);
+                    g[jt][e] = (jc & 1) ? p_odd[(jc / 2) * PD] : p_even[(jc / 2) * PD];
+                }
+#pragma unroll
+            for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) s_acc[jt][e] = E::pick(g[jt][e], (e & 1) ? sel_odd : sel_even);
         } else {
             s_acc[0] = zero16;
             s_acc[1] = zero16;
@@ -809,9 +832,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         cphase = cphase == 2 * BN ? 0 : cphase + BN;
         // all LDS reads of the half in flight together, then the conversions, then the score MFMAs (they share the
         // matrix pipe of this half with the position wave of the SIMD)
-        __builtin_amdgcn_sched_group_barrier(0x200, 4, 0);    // K / V stores
-        __builtin_amdgcn_sched_group_barrier(0x100, 36, 0);   // ring fragments and P' elements
-        __builtin_amdgcn_sched_group_barrier(0x002, 32, 0);   // conversions
+        store_kv(s & 1, s + 2 < nsteps);  // (in the last step the key buffers already take the next tile's keys)
 #pragma unroll
         for (int c = 0; c < 4; ++c)
 #pragma unroll
