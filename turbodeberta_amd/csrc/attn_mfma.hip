@@ -123,7 +123,7 @@ __device__ __forceinline__ void phase_barrier() {
     __builtin_amdgcn_sched_barrier(0);
 }
 
-template <bool HAS_C2P, bool HAS_P2C, int DT>
+template <bool HAS_C2P, bool HAS_P2C, int DT, bool FARZ>
 __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelParams p, const int nblocks) {
     using E = Elem<DT>;
     using ET = typename E::T;
@@ -340,6 +340,15 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     auto pq_of = [&](const Tile& t) { return HAS_P2C ? static_cast<const uint16_t*>(p.pq) + int64_t(t.head) * p.pqs_h : nullptr; };
 
     auto next_tile = [&](const Tile& t) { return balanced ? next_balanced(t) : find_tile(t.vb + gridDim.x); };
+    // A key step is "far" when its whole window of relative positions maps to ONE table row (delta is monotone in r, so
+    // its two ends decide): beyond max_relative_positions on either side, which is most of a long sequence.  Then the
+    // c2p term is one value per query and the p2c term one value per key, and the step needs no window products, no
+    // ring and no scratch.  Step t of the tile that starts at query row r0: window r0 - 64t - 63 .. + 190.
+    auto far_at = [&](int r0, int t) {
+        if (!HAS_POS || !FARZ) return false;
+        const int b = r0 - BN * t - (BN - 1);
+        return delta_of(b) == delta_of(b + WIN - 2);
+    };
 
     Tile cur = balanced ? first_balanced() : find_tile(blockIdx.x);
     if (cur.vb < 0) return;
@@ -552,6 +561,25 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
                 else if (w == 1) pack_p(chain(fq[1], kb[0]), ppk[2]);
             }
         };
+        // Far step: every window row is the same table row, so any fragment tile will do.  Row 0 of K_r'.Q^T is the one
+        // c2p value of each query and row 0 of Q_r'.K^T the one p2c value of each key (position waves 0 and 1 take one key
+        // tile each); register 0 of the lower half-wave holds row 0.  Both go to the (idle) scratch as fp32: 64 key values,
+        // then 128 query values.
+        float far_c = 0.f, far_d = 0.f;
+        auto far_products = [&]() {
+            if (HAS_C2P) far_c = chain(fr[0], qb)[0];
+            if (HAS_P2C) {
+                if (w == 0) far_d = chain(fq[0], kb[0])[0];
+                else if (w == 1) far_d = chain(fq[0], kb[1])[0];
+            }
+        };
+        auto put_far = [&]() {
+            float* const fv = reinterpret_cast<float*>(sm.p);
+            if (hh == 0) {
+                if (HAS_C2P) fv[BN + 32 * w + il] = far_c;
+                if (HAS_P2C && w < 2) fv[32 * w + il] = far_d;
+            }
+        };
         // Ring slot of the group (rt, a) of batch t: key 64t + ckey - 32rt - 8a with ckey = 60 + 4il - 4hh; `phase` is
         // 64t mod 192.
         uint16_t* const crow = sm.c + (32 * w + il) * CRS;
@@ -641,6 +669,9 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
             dl_step[s1][0] = dl_cold[s1][0];
             dl_step[s1][1] = dl_cold[s1][1];
         }
+        // near flags (not far) of steps 0, 1, 2 of the tile about to open; c2p batch t is needed when one of the steps
+        // t, t+1, t+2 -- the steps its keys 64t + 4n .. 64t + 63 + 4n fall into -- is near
+        bool near0 = !far_at(cur.row0, 0), near1 = !far_at(cur.row0, 1), near2 = !far_at(cur.row0, 2);
         phase_barrier();                  // first stage of the first tile is in LDS
         while (true) {
             bind_tables();
@@ -651,17 +682,26 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
             dl_next[1] = dl_step[0][1];
             fetch();                      // window rows of step 1; they arrive under the products of step 0
             load_fp(0, 0);
-            load_fr(0, w + 2 * BN);
-            products_c();
-            put_c(BN);                    // batch -2: phase (-128) mod 192
-            load_fr(0, w + BN);
-            products_c();
-            put_c(2 * BN);                // batch -1
-            load_fr(0, w);
-            products_c();
-            put_c(0);                     // batch 0
-            products_p();
-            put_p();
+            if (near0 || near1 || near2) {
+                load_fr(0, w + 2 * BN);
+                products_c();
+                put_c(BN);                // batch -2: phase (-128) mod 192
+                load_fr(0, w + BN);
+                products_c();
+                put_c(2 * BN);            // batch -1
+                load_fr(0, w);
+                products_c();
+                put_c(0);                 // batch 0
+            } else {
+                load_fr(0, w);
+            }
+            if (near0) {
+                products_p();
+                put_p();
+            } else {
+                far_products();
+                put_far();
+            }
             phase_barrier();              // every position wave has read its fragments of step 0
             store(off1);
             dl_next[0] = dl_step[1][0];
@@ -681,11 +721,15 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
 
             int off2 = prev_off(off1);    // ring offset of step s+2
             int phase = BN;               // ring phase of batch s+1
+            bool n1 = near1, n2 = near2, n3 = !far_at(row0, 3);      // near flags of steps s+1, s+2, s+3
             auto pos_step = [&](int s, auto tail_tag) {
                 constexpr bool TAIL = decltype(tail_tag)::value;   // step nsteps-2: no step s+2 to prepare
+                const bool batch = n1 || n2 || n3;                 // c2p batch s+1 has a reader
+                const bool n4 = !far_at(row0, s + 4);              // (a scalar read, used in the next step)
                 phase_barrier();          // position terms of step s complete
-                products_c();             // of step s+1, into registers; issued first: the wait for the
-                products_p();
+                if (batch) products_c();  // of step s+1, into registers; issued first: the wait for the
+                if (n1) products_p();
+                else far_products();
                 __builtin_amdgcn_sched_barrier(0);  // prefetched global data then passes under the MFMAs
                 if (!TAIL) {
                     store(off2);          // new window rows of step s+2
@@ -693,8 +737,9 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
                     fetch_delta(s + 4);
                 }
                 phase_barrier();          // score waves are done with the ring slots and the scratch; the staged tiles are visible
-                put_c(phase);             // of step s+1
-                put_p();
+                if (batch) put_c(phase);  // of step s+1
+                if (n1) put_p();
+                else put_far();
                 if (!TAIL) {
                     load_fp(off2, s & 1); // of step s+2
                     load_fr(off2, w);
@@ -703,6 +748,9 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
                 }
                 off2 = prev_off(off2);
                 phase = next_phase(phase);
+                n1 = n2;
+                n2 = n3;
+                n3 = n4;
             };
             if (nsteps >= 2) {
                 for (int s = 0; s + 2 < nsteps; ++s) pos_step(s, std::false_type{});
@@ -714,6 +762,9 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
             // registers are free, so the next tile moves in; the barrier that ends this half is also the barrier
             // after which the next tile's first stage is in LDS.
             phase_barrier();
+            near0 = !far_at(nxt.row0, 0);
+            near1 = !far_at(nxt.row0, 1);
+            near2 = !far_at(nxt.row0, 2);
             read_stage(nxt);
             load_q(qb, nxt);              // (the last products of this tile have read the old fragments)
             if (nxt.vb >= 0) write_stage();
@@ -782,6 +833,8 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     nxt.cost = 0;
     nxt.tok0 = 0;
     int cphase = 0;                       // ring slot of the first key of the step: 64s mod 192
+    bool far_cur = false;                 // whether the step about to run is far; far_open: step 0 of the tile to open
+    bool far_open = far_at(cur.row0, 0);
     const uint16_t* const crow = sm.c + (32 * w + il) * CRS + 8 * hh;
     // One key step.  MASKED: the step reaches past the end of the sequence (only the last step can).
     auto key_step = [&](int s, auto masked_tag) {
@@ -792,15 +845,32 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         //      position terms of step s: c2p as four B operands of 16 keys each, straight out of the ring (keys
         //      64s .. 64s+63 never straddle its wrap), p2c element by element: (key jj, query n) takes
         //      P'[jj][w + 4n + 63 - jj], converted to fp32 into what becomes the initial score accumulator ----------
+        const bool far_nxt = far_at(row0, s + 1);     // (two scalar reads, used at the end of the step)
         X8 cf[2][2];
-        if (HAS_C2P) {
+        if (HAS_C2P && !far_cur) {
 #pragma unroll
             for (int jt = 0; jt < 2; ++jt)
 #pragma unroll
                 for (int c2 = 0; c2 < 2; ++c2) cf[jt][c2] = *reinterpret_cast<const X8*>(crow + cphase + 32 * jt + 16 * c2);
         }
         f32x16 s_acc[2];
-        if (HAS_P2C) {
+        float cadd = 0.f;                 // far step: the c2p value of this lane's query, added when the scores are scaled
+        if (far_cur) {
+            // one p2c value per key (fp32, the same for every query): the initial accumulator; one c2p value per query
+            const float* const fv = reinterpret_cast<const float*>(sm.p);
+            if (HAS_C2P) cadd = fv[BN + 32 * w + il];
+#pragma unroll
+            for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+                for (int a = 0; a < 4; ++a) {
+                    float4 d = float4{0.f, 0.f, 0.f, 0.f};
+                    if (HAS_P2C) d = *reinterpret_cast<const float4*>(fv + 32 * jt + 8 * a + 4 * hh);
+                    s_acc[jt][4 * a] = d.x;
+                    s_acc[jt][4 * a + 1] = d.y;
+                    s_acc[jt][4 * a + 2] = d.z;
+                    s_acc[jt][4 * a + 3] = d.w;
+                }
+        } else if (HAS_P2C) {
             // Element (key jc, query n) sits at 16-bit index X + jc * (PS - 1), X = w + 63 + 4n: from one key to the next
             // the index moves by an odd amount, so the element alternates between the low and the high half of its
             // dword with the parity of jc, starting from the parity of w + 1 -- the same for every lane, because the
@@ -837,7 +907,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         for (int c = 0; c < 4; ++c)
 #pragma unroll
             for (int jt = 0; jt < 2; ++jt) s_acc[jt] = E::mfma(kf[jt][c], qb[c], s_acc[jt]);
-        if (HAS_C2P) {
+        if (HAS_C2P && !far_cur) {
 #pragma unroll
             for (int c2 = 0; c2 < 2; ++c2)
 #pragma unroll
@@ -847,7 +917,10 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         phase_barrier();                  // ring slots and scratch are free again; keys of step s+1 and values of step s are staged
 
         // ---- half B ---------------------------------------------------------------------------------------------
-        if (s + 1 == nsteps) load_q(qb, nxt);   // last step: the Q fragments of the next tile travel from here on
+        if (s + 1 == nsteps) {            // last step: the Q fragments of the next tile travel from here on
+            load_q(qb, nxt);
+            far_open = far_at(nxt.row0, 0);
+        }
         if (s + 1 < nsteps) fetch_kv(s + 3, s + 1);   // for the next half A (nothing left to fetch in the last step)
         // V^T fragments through the transposing LDS read: the lane provides the address of 4 dims of one key
         X8 vf[2][2][2];               // [key tile][16-key chunk][dim tile]
@@ -882,7 +955,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         for (int jt = 0; jt < 2; ++jt)
 #pragma unroll
             for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s_acc[jt][e]);
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        mx = fmaxf(mx, __shfl_xor(mx, 32)) + cadd;
         // The running maximum is only raised (and the accumulators rescaled) when some row of the wave exceeds it
         // by more than 2^8; until then probabilities of this step may be as large as 256, which bf16 and the fp32
         // sums carry exactly as well.  (First step: m_run = -inf always triggers, alpha = 0.)
@@ -896,7 +969,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
                 for (int e = 0; e < 16; ++e) o_acc[t][e] *= alpha;
             m_run = m_new;
         }
-        const float mc = m_run * c_exp;
+        const float mc = (m_run - cadd) * c_exp;
         float psum = 0.f;
 #pragma unroll
         for (int jt = 0; jt < 2; ++jt)
@@ -918,6 +991,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
                     o_acc[dt] = E::mfma(vf[jt][c][dt], pb, o_acc[dt]);
             }
         l_run += psum;
+        far_cur = far_nxt;
     };
 
     // Opening of a tile, after its first barrier (first stage in LDS).  Everything that reads global memory is
@@ -937,6 +1011,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
                 for (int a = 0; a < 2; ++a) *reinterpret_cast<u32x4*>(o_ptr + 32 * dt + 16 * a) = o_out[dt][a];
         }
         cphase = 0;
+        far_cur = far_open;
         phase_barrier();                  // the two opening barriers of the position waves
         phase_barrier();
         // the tile after this one is looked up while the position waves get step 1 ready
@@ -1016,7 +1091,8 @@ namespace {
 // Per-device launch facts, looked up once per device under a lock: CU count (rounded down to the 8 XCDs the block
 // ids are dealt over) and, per kernel instance, whether its dynamic-LDS limit has been raised on that device.
 constexpr int kMaxDevices = 64;
-constexpr int kInstances = 8;
+constexpr int FAR_MIN_LEN = 1024;
+constexpr int kInstances = 16;
 std::mutex g_dev_mutex;
 int g_cus[kMaxDevices] = {0};
 bool g_attr_set[kMaxDevices][kInstances] = {{false}};
@@ -1048,10 +1124,15 @@ hipError_t tdb_launch_mfma(const TdbKernelParams& whole, int dtype, hipStream_t 
     if (e != hipSuccess) return e;
     if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
     const bool c2p = p.pk != nullptr, p2c = p.pq != nullptr;
-    const int instance = (dtype == TDB_F16 ? 4 : 0) + (c2p ? 2 : 0) + (p2c ? 1 : 0);
+    // Far key steps only exist in sequences longer than the table's reach; the instance that looks for them carries
+    // both step bodies and is a little slower on steps that are not far, so short launches take the one without.
+    const bool farz = (c2p || p2c) && p.L >= FAR_MIN_LEN;
+    const int instance = (farz ? 8 : 0) + (dtype == TDB_F16 ? 4 : 0) + (c2p ? 2 : 0) + (p2c ? 1 : 0);
     const size_t smem = sizeof(Smem);
     const void* fn = nullptr;
-#define TDB_PICK(A, B, T) fn = reinterpret_cast<const void*>(&attn_mfma_kernel<A, B, T>)
+#define TDB_PICK(A, B, T)                                                                 \
+    fn = farz ? reinterpret_cast<const void*>(&attn_mfma_kernel<A, B, T, true>)           \
+              : reinterpret_cast<const void*>(&attn_mfma_kernel<A, B, T, false>)
 #define TDB_PICK_T(T)                                      \
     do {                                                   \
         if (c2p && p2c) TDB_PICK(true, true, T);           \
