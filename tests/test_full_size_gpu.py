@@ -197,6 +197,55 @@ def test_config5_packed_variant_8_sequences():
     assert_close_bf16(out[s:e][:, hs].permute(1, 0, 2), ref, "config 5 packed variant vs oracle", tol=1e-2)
 
 
+def _rows_in_float64(q, k, v, pk, pq, n, rows):
+    """Attention output of single query rows of one sequence ([n, H, D] tensors on the GPU), in float64:
+    scores (q_i.k_j + q_i.K_r[delta(i-j)] + k_j.Q_r[delta(i-j)]) * SCALE over all n keys, softmax, times v
+    (modeling_deberta_v2.py:318-343 with both position terms); delta from the oracle's table."""
+    delta = torch.from_numpy(O.delta_table(n, BUCKETS, MAX_REL).astype(np.int64)).to(DEV)           # entry r + n - 1
+    qd, kd, vd, pkd, pqd = (t.double() for t in (q, k, v, pk, pq))
+    out = []
+    for i in rows:
+        d = delta[i - torch.arange(n, device=DEV) + n - 1]                                            # [n]
+        c2p = torch.einsum("hd,hnd->nh", qd[i], pkd[:, d])                                            # q_i . K_r[delta]
+        p2c = torch.einsum("nhd,hnd->nh", kd, pqd[:, d])                                              # k_j . Q_r[delta]
+        sc = (torch.einsum("hd,nhd->nh", qd[i], kd) + c2p + p2c) * SCALE
+        out.append(torch.einsum("nh,nhd->hd", torch.softmax(sc, dim=0), vd))
+    return torch.stack(out)                                                                           # [rows, H, D]
+
+
+def test_packed_sequence_of_131072_tokens():
+    """One sequence of 2^17 tokens packed with a short one (2 heads): 1024 query tiles of 2048 key steps each, dealt
+    by cost over all workgroups -- the tile walk's cost coordinates pass 2^31 / 64 here -- and almost every key step
+    takes the far path.  Sampled query rows of the long sequence against the float64 row formula (itself compared
+    with the oracle on the short sequence), every row of the short sequence against the oracle."""
+    heads, lengths = 2, [131072, 300]
+    T = sum(lengths)
+    g = torch.Generator(device=DEV).manual_seed(17)
+    mk = lambda *s: torch.randn(*s, generator=g, device=DEV)
+    q, k, v = (mk(T, heads, D).bfloat16() for _ in range(3))
+    pk, pq = (mk(heads, 2 * SPAN, D).bfloat16() for _ in range(2))
+    cu = torch.tensor([0, lengths[0], T], dtype=torch.int32, device=DEV)
+    print("[case] packed 131072 + 300 tokens, 2 heads", flush=True)
+    out = flash_attention_with_disentangled_varlen(q, k, v, None, None, cu, cu, lengths[0], lengths[0], False, SCALE,
+                                                   BUCKETS, MAX_REL, pos_key_layer=pk, pos_query_layer=pq)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out.float()).all()
+    n = lengths[0]
+    rows = [0, 1, 127, 128, 511, 600, 65535, 65536, 100003, n - 129, n - 2, n - 1]
+    want = _rows_in_float64(q[:n], k[:n], v[:n], pk, pq, n, rows)
+    # an average over ~10^5 values of size 1 is small: the tolerance is relative to the largest expected entry
+    assert_close_bf16(out[rows], want, "2^17-token sequence, sampled rows", tol=0.02 * want.abs().max().item())
+    # the short sequence: oracle, and the row formula against the oracle
+    s = slice(n, T)
+    f = lambda t: t[s].permute(1, 0, 2)[None].float().cpu()
+    ref = O.attention(f(q), f(k), f(v), pk.float().cpu(), pq.float().cpu(), None,
+                      position_buckets=BUCKETS, max_relative_positions=MAX_REL)[0].permute(1, 0, 2)     # [300, H, D]
+    assert_close_bf16(out[s], ref, "short sequence packed behind it", tol=1e-2)
+    few = [0, 150, 299]
+    mine = _rows_in_float64(q[s], k[s], v[s], pk, pq, lengths[1], few)
+    assert (mine.float().cpu() - ref[few]).abs().max().item() <= 1e-4
+
+
 def test_persistent_tile_walk_mixed_lengths():
     """More tiles than workgroups, with everything a persistent workgroup can meet on its list: single-step tiles
     (length <= 64), tiles with only padded rows (in the middle and at the end of a list), a sequence of length 0,
