@@ -561,18 +561,25 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
                 if (HAS_P2C) pre_qr[n] = __builtin_amdgcn_raw_buffer_load_b128(pq_rsrc, dl_next[n] * pqs_b + sch * 16, 0, 0);
             }
         };
-        auto fetch_delta = [&](int s) {        // delta of the 64 new window rows of key step s
+        // delta of the 64 new window rows of key step s: relative positions row0 - 64s - 63 + srow (+ 32).  Read through
+        // a buffer over the table: positions outside it (they belong to keys or queries that do not exist) read as 0,
+        // a valid row, with no clamping arithmetic.
+        const __amdgpu_buffer_rsrc_t lut_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<int*>(p.lut), 0, (lut_max + 1) * 4, RSRC_FLAGS);
+        const int srow4 = srow * 4;
+        auto fetch_delta = [&](int s) {
             if (HAS_POS) {
-#pragma unroll
-                for (int n = 0; n < 2; ++n) dl_next[n] = delta_of(row0 - BN * s - (BN - 1) + srow + 32 * n);
+                const int off = srow4 + (row0 - BN * s - (BN - 1) + p.lut_half) * 4;
+                dl_next[0] = __builtin_amdgcn_raw_buffer_load_b32(lut_rsrc, off, 0, 0);
+                dl_next[1] = __builtin_amdgcn_raw_buffer_load_b32(lut_rsrc, off + 128, 0, 0);
             }
         };
+        const int stage_el = srow * RS + sch * 8;
         auto store = [&](int o) {              // registers -> LDS: window rows at ring offset o
+            const int el = stage_el + o * RS;  // (o is wave-uniform: one vector add, the row inside the step is an immediate)
 #pragma unroll
             for (int n = 0; n < 2; ++n) {
-                const int r = srow + 32 * n;
-                if (HAS_C2P) *reinterpret_cast<u32x4*>(&sm.kr[(o + r) * RS + sch * 8]) = pre_kr[n];
-                if (HAS_P2C) *reinterpret_cast<u32x4*>(&sm.qr[(o + r) * RS + sch * 8]) = pre_qr[n];
+                if (HAS_C2P) *reinterpret_cast<u32x4*>(&sm.kr[el + 32 * n * RS]) = pre_kr[n];
+                if (HAS_P2C) *reinterpret_cast<u32x4*>(&sm.qr[el + 32 * n * RS]) = pre_qr[n];
             }
         };
         // Position products of one key step, in three stages that the pipeline places in different halves:
@@ -672,14 +679,18 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         const int ckey = 60 + 4 * il - 4 * hh;
         auto put_c = [&](int phase) {
             if (HAS_C2P) {
+                // slot of group (rt, a): y = cb - 32rt - 8a, minus 192 once y reaches 192 -- two base addresses per
+                // step, one compare and one select per store, the distance inside the group as an immediate
                 const int cb = phase + ckey;                    // 56 .. 312
+                uint16_t* const flat = crow + cb - 56;
+                uint16_t* const wrapped = flat - CRING;
 #pragma unroll
                 for (int rt = 0; rt < 2; ++rt)
 #pragma unroll
                     for (int a = 0; a < 4; ++a) {
-                        const int y = cb - 32 * rt - 8 * a;
-                        const int slot = y >= CRING ? y - CRING : y;
-                        *reinterpret_cast<u32x2*>(crow + slot) = cpk[rt][a];
+                        const int d = 32 * rt + 8 * a;
+                        uint16_t* const base = cb >= CRING + d ? wrapped : flat;
+                        *reinterpret_cast<u32x2*>(base + 56 - d) = cpk[rt][a];
                     }
             }
         };
@@ -924,6 +935,16 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     bool far_open = far_at(cur.row0, 0);
     const uint16_t* const crow = sm.c + (32 * w + il) * CRS + 8 * hh;
     // One key step.  MASKED: the step reaches past the end of the sequence (only the last step can).
+    // The value lane ^ 32 holds.  A lane swap in the vector ALU: a shuffle would travel through the LDS queue, behind
+    // the transposing reads of this wave and the result stores of the position waves, with the softmax waiting for it.
+    // Swapping the upper half of one copy with the lower half of another leaves {own, partner} in the two results
+    // (in an order that depends on the half, which a maximum or a sum does not care about).
+    auto both_halves = [](float x, float& a, float& b) {
+        const uint32_t u = __builtin_bit_cast(uint32_t, x);
+        const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+        a = __builtin_bit_cast(float, uint32_t(r[0]));
+        b = __builtin_bit_cast(float, uint32_t(r[1]));
+    };
     auto key_step = [&](int s, auto masked_tag) {
         constexpr bool MASKED = decltype(masked_tag)::value;
         phase_barrier();                  // position terms of step s complete
@@ -1047,7 +1068,11 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         for (int jt = 0; jt < 2; ++jt)
 #pragma unroll
             for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s_acc[jt][e]);
-        mx = fmaxf(mx, __shfl_xor(mx, 32)) + cadd;
+        {
+            float own_or_partner, partner_or_own;
+            both_halves(mx, own_or_partner, partner_or_own);
+            mx = fmaxf(own_or_partner, partner_or_own) + cadd;
+        }
         // The running maximum is only raised (and the accumulators rescaled) when some row of the wave exceeds it
         // by more than 2^8; until then probabilities of this step may be as large as 256, which bf16 and the fp32
         // sums carry exactly as well.  (First step: m_run = -inf always triggers, alpha = 0.)
@@ -1115,7 +1140,9 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     // eight consecutive d (lane half hh keeps the blocks a = 2*a2 + hh), so a row goes out in 16-byte stores.
     auto close_tile = [&]() {
         const int qi = row0 + 4 * il + w;
-        const float l_tot = l_run + __shfl_xor(l_run, 32);
+        float l_a, l_b;
+        both_halves(l_run, l_a, l_b);
+        const float l_tot = l_a + l_b;
         const float inv = 1.f / l_tot;
         const bool live = qi < len;
         o_write = qi < row0 + rows_here;
