@@ -133,7 +133,11 @@ __device__ __forceinline__ void phase_barrier() {
     __builtin_amdgcn_sched_barrier(0);
 }
 
-template <bool HAS_C2P, bool HAS_P2C, int DT, bool FARZ>
+// Template parameters: which position terms exist, the element type, whether far key steps are looked for, and the
+// layout (VARLEN: packed sequences).  The layout is a compile-time fact because the tile bookkeeping of the two layouts
+// has nothing in common: with both compiled into one instance, the unused one still cost scalar registers (spilled
+// into vector lanes and reloaded in the step loops) and several hundred scalar instructions per tile.
+template <bool HAS_C2P, bool HAS_P2C, int DT, bool FARZ, bool VARLEN>
 __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelParams p, const int nblocks) {
     using E = Elem<DT>;
     using ET = typename E::T;
@@ -157,7 +161,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     // Virtual block -> (tile, head): consecutive ids go round-robin over the 8 XCDs, each with its own L2; ids are
     // regrouped so that XCD_GROUP tiles that are neighbours along the query axis -- the tiles that read the same K
     // and V -- run on one XCD and fetch K / V from HBM once instead of once each.
-    const int tiles_x = p.varlen ? p.total / BM + p.B : p.B * ((p.L + BM - 1) / BM);
+    const int tiles_x = VARLEN ? p.total / BM + p.B : p.B * ((p.L + BM - 1) / BM);
     const int lut_max = 2 * p.lut_half;
     auto delta_of = [&](int r) { return p.lut[min(max(r + p.lut_half, 0), lut_max)]; };
 
@@ -203,10 +207,10 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     // none, so teams are pairs.)  Cost coordinates are 64-bit: one sequence of 2^20 tokens alone costs 2^30.  The
     // state of the deal (next tile of the list, cost per member) lives in LDS, one copy per wave: it is touched once
     // per tile and would otherwise occupy registers all through the key steps.
-    const bool balanced = p.varlen && p.B <= 64;
+    const bool balanced = VARLEN && p.B <= 64;
     {
         int n = p.L, lo = 0;
-        if (p.varlen) {
+        if (VARLEN) {
             lo = p.cu_seqlens[min(l, p.B)];
             const int hi = p.cu_seqlens[min(l + 1, p.B)];
             n = hi - lo;
@@ -227,7 +231,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     }
     // tile_id -> (sequence, first row, valid length, first token): same map as tdb_locate_tile
     auto locate = [&](int tile_id, int& bb, int& r0, int& ln, int64_t& t0) {
-        if (!p.varlen) {
+        if (!VARLEN) {
             const int tiles = (p.L + BM - 1) / BM;
             bb = tile_id / tiles;
             r0 = (tile_id - bb * tiles) * BM;
@@ -403,8 +407,8 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
             int64_t t0;
             if (!locate(tile_id, bb, r0, ln, t0)) continue;
             if (r0 >= ln) {
-                uint16_t* Oz = static_cast<uint16_t*>(p.o) + (p.varlen ? t0 * p.os_l : int64_t(bb) * p.os_b) + int64_t(hd) * p.os_h;
-                const int rows = min(BM, (p.varlen ? ln : p.L) - r0);
+                uint16_t* Oz = static_cast<uint16_t*>(p.o) + (VARLEN ? t0 * p.os_l : int64_t(bb) * p.os_b) + int64_t(hd) * p.os_h;
+                const int rows = min(BM, (VARLEN ? ln : p.L) - r0);
                 for (int idx = tid; idx < rows * (D / 8); idx += NTHREADS)
                     *reinterpret_cast<u32x4*>(Oz + int64_t(r0 + (idx >> 3)) * p.os_l + (idx & 7) * 8) = u32x4{0, 0, 0, 0};
                 continue;
@@ -420,7 +424,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         return t;
     };
     auto k_of = [&](const Tile& t) {
-        return static_cast<const uint16_t*>(p.k) + (p.varlen ? t.tok0 * p.ks_l : int64_t(t.b) * p.ks_b) + int64_t(t.head) * p.ks_h;
+        return static_cast<const uint16_t*>(p.k) + (VARLEN ? t.tok0 * p.ks_l : int64_t(t.b) * p.ks_b) + int64_t(t.head) * p.ks_h;
     };
     auto pk_of = [&](const Tile& t) { return HAS_C2P ? static_cast<const uint16_t*>(p.pk) + int64_t(t.head) * p.pks_h : nullptr; };
     auto pq_of = [&](const Tile& t) { return HAS_P2C ? static_cast<const uint16_t*>(p.pq) + int64_t(t.head) * p.pqs_h : nullptr; };
@@ -477,11 +481,11 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         len = t.len;
         nsteps = (len + BN - 1) / BN;
         nfull = len / BN;                 // steps that need no key mask
-        rows_here = min(BM, (p.varlen ? len : p.L) - row0);   // rows of this tile that exist in memory
-        Q = static_cast<const uint16_t*>(p.q) + (p.varlen ? t.tok0 * p.qs_l : int64_t(t.b) * p.qs_b) + int64_t(t.head) * p.qs_h;
+        rows_here = min(BM, (VARLEN ? len : p.L) - row0);   // rows of this tile that exist in memory
+        Q = static_cast<const uint16_t*>(p.q) + (VARLEN ? t.tok0 * p.qs_l : int64_t(t.b) * p.qs_b) + int64_t(t.head) * p.qs_h;
         K = k_of(t);
-        V = static_cast<const uint16_t*>(p.v) + (p.varlen ? t.tok0 * p.vs_l : int64_t(t.b) * p.vs_b) + int64_t(t.head) * p.vs_h;
-        O = static_cast<uint16_t*>(p.o) + (p.varlen ? t.tok0 * p.os_l : int64_t(t.b) * p.os_b) + int64_t(t.head) * p.os_h;
+        V = static_cast<const uint16_t*>(p.v) + (VARLEN ? t.tok0 * p.vs_l : int64_t(t.b) * p.vs_b) + int64_t(t.head) * p.vs_h;
+        O = static_cast<uint16_t*>(p.o) + (VARLEN ? t.tok0 * p.os_l : int64_t(t.b) * p.os_b) + int64_t(t.head) * p.os_h;
         PK = pk_of(t);
         PQ = pq_of(t);
     };
@@ -490,7 +494,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     // Q^T fragments of query block w: B operand of S^T = K.Q^T (score wave) and of C'^T = K_r'.Q^T (position wave)
     X8 qb[4];
     auto load_q = [&](X8 (&dst)[4], const Tile& t) {
-        const uint16_t* Qt = static_cast<const uint16_t*>(p.q) + (p.varlen ? t.tok0 * p.qs_l : int64_t(t.b) * p.qs_b) + int64_t(t.head) * p.qs_h;
+        const uint16_t* Qt = static_cast<const uint16_t*>(p.q) + (VARLEN ? t.tok0 * p.qs_l : int64_t(t.b) * p.qs_b) + int64_t(t.head) * p.qs_h;
         const int qrow = t.row0 + 4 * il + w;
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
@@ -1042,7 +1046,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
             // keys of step 2 and values of step 0 of the next tile: its first half A stores them, and a first touch of
             // a new sequence takes longer than the opening of a tile lasts
             if (nxt.vb >= 0)
-                fetch_kv_from(k_of(nxt), static_cast<const uint16_t*>(p.v) + (p.varlen ? nxt.tok0 * p.vs_l : int64_t(nxt.b) * p.vs_b) + int64_t(nxt.head) * p.vs_h,
+                fetch_kv_from(k_of(nxt), static_cast<const uint16_t*>(p.v) + (VARLEN ? nxt.tok0 * p.vs_l : int64_t(nxt.b) * p.vs_b) + int64_t(nxt.head) * p.vs_h,
                               nxt.len, 2, 0);
         }
         if (s + 1 < nsteps) fetch_kv(s + 3, s + 1);   // for the next half A (nothing left to fetch in the last step)
@@ -1225,7 +1229,7 @@ namespace {
 // ids are dealt over) and, per kernel instance, whether its dynamic-LDS limit has been raised on that device.
 constexpr int kMaxDevices = 64;
 constexpr int FAR_MIN_LEN = 1024;
-constexpr int kInstances = 16;
+constexpr int kInstances = 32;
 std::mutex g_dev_mutex;
 int g_cus[kMaxDevices] = {0};
 bool g_attr_set[kMaxDevices][kInstances] = {{false}};
@@ -1260,12 +1264,14 @@ hipError_t tdb_launch_mfma(const TdbKernelParams& whole, int dtype, hipStream_t 
     // Far key steps only exist in sequences longer than the table's reach; the instance that looks for them carries
     // both step bodies and is a little slower on steps that are not far, so short launches take the one without.
     const bool farz = (c2p || p2c) && p.L >= FAR_MIN_LEN;
-    const int instance = (farz ? 8 : 0) + (dtype == TDB_F16 ? 4 : 0) + (c2p ? 2 : 0) + (p2c ? 1 : 0);
+    const int instance = (p.varlen ? 16 : 0) + (farz ? 8 : 0) + (dtype == TDB_F16 ? 4 : 0) + (c2p ? 2 : 0) + (p2c ? 1 : 0);
     const size_t smem = sizeof(Smem);
     const void* fn = nullptr;
-#define TDB_PICK(A, B, T)                                                                 \
-    fn = farz ? reinterpret_cast<const void*>(&attn_mfma_kernel<A, B, T, true>)           \
-              : reinterpret_cast<const void*>(&attn_mfma_kernel<A, B, T, false>)
+#define TDB_PICK(A, B, T)                                                                                        \
+    fn = farz ? (p.varlen ? reinterpret_cast<const void*>(&attn_mfma_kernel<A, B, T, true, true>)                \
+                          : reinterpret_cast<const void*>(&attn_mfma_kernel<A, B, T, true, false>))              \
+              : (p.varlen ? reinterpret_cast<const void*>(&attn_mfma_kernel<A, B, T, false, true>)               \
+                          : reinterpret_cast<const void*>(&attn_mfma_kernel<A, B, T, false, false>))
 #define TDB_PICK_T(T)                                      \
     do {                                                   \
         if (c2p && p2c) TDB_PICK(true, true, T);           \
