@@ -207,7 +207,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     // none, so teams are pairs.)  Cost coordinates are 64-bit: one sequence of 2^20 tokens alone costs 2^30.  The
     // state of the deal (next tile of the list, cost per member) lives in LDS, one copy per wave: it is touched once
     // per tile and would otherwise occupy registers all through the key steps.
-    const bool balanced = VARLEN && p.B <= 64;
+    constexpr bool balanced = VARLEN;     // (the launcher never hands more than 64 packed sequences to one launch)
     {
         int n = p.L, lo = 0;
         if (VARLEN) {
@@ -429,7 +429,10 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     auto pk_of = [&](const Tile& t) { return HAS_C2P ? static_cast<const uint16_t*>(p.pk) + int64_t(t.head) * p.pks_h : nullptr; };
     auto pq_of = [&](const Tile& t) { return HAS_P2C ? static_cast<const uint16_t*>(p.pq) + int64_t(t.head) * p.pqs_h : nullptr; };
 
-    auto next_tile = [&](const Tile& t) { return balanced ? take() : find_tile(t.vb + gridDim.x); };
+    auto next_tile = [&](const Tile& t) {
+        if constexpr (balanced) return take();
+        else return find_tile(t.vb + gridDim.x);
+    };
     // A key step is "far" when its whole window of relative positions maps to ONE table row (delta is monotone in r, so
     // its two ends decide): beyond max_relative_positions on either side, which is most of a long sequence.  Then the
     // c2p term is one value per query and the p2c term one value per key, and the step needs no window products, no
@@ -440,7 +443,9 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         return delta_of(b) == delta_of(b + WIN - 2);
     };
 
-    Tile cur = balanced ? first_balanced() : find_tile(blockIdx.x);
+    Tile cur;
+    if constexpr (balanced) cur = first_balanced();
+    else cur = find_tile(blockIdx.x);
     if (cur.vb < 0) return;
 
     // ---- pipeline of one tile -----------------------------------------------------------------------------------
