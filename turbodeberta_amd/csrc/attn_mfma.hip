@@ -190,10 +190,8 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     };
     auto tiles_of = [](int n) { return (n + BM - 1) / BM; };
     auto cost_of = [](int n) { return int64_t(8 * ((n + BN - 1) / BN) + 13); };
-    // Packed launches of up to 64 sequences (the launcher splits larger batches, so that is every packed launch it
-    // makes; a larger one would take the strided walk with the tile numbering of `locate`) use a cost-balanced walk
-    // instead of the strided one: tiles differ in
-    // length by up to 8x, so a TEAM of workgroups takes a CONTIGUOUS range of the tile list (heads outermost, then
+    // Packed launches (at most 64 sequences: the launcher splits larger batches) use a cost-balanced walk instead of
+    // the strided one of the fixed layout: tiles differ in length by up to 8x, so a TEAM of workgroups takes a CONTIGUOUS range of the tile list (heads outermost, then
     // sequences, then the query tiles of a sequence) whose summed cost is its share of the total.  The cost of a tile
     // is 8 * (its key steps) + 13, in eighths of a key step (13: what opening a tile costs).  Every wave derives the
     // same ranges from the sequence boundaries; a tile belongs to the team whose cost interval holds the tile's
@@ -207,7 +205,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     // none, so teams are pairs.)  Cost coordinates are 64-bit: one sequence of 2^20 tokens alone costs 2^30.  The
     // state of the deal (next tile of the list, cost per member) lives in LDS, one copy per wave: it is touched once
     // per tile and would otherwise occupy registers all through the key steps.
-    constexpr bool balanced = VARLEN;     // (the launcher never hands more than 64 packed sequences to one launch)
+    constexpr bool balanced = VARLEN;
     {
         int n = p.L, lo = 0;
         if (VARLEN) {
@@ -229,48 +227,14 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         sm.seq_lo[l] = lo;
         sm.seq_pre[l] = pre;
     }
-    // tile_id -> (sequence, first row, valid length, first token): same map as tdb_locate_tile
+    // fixed layout: tile_id -> (sequence, first row, valid length); same map as tdb_locate_tile
     auto locate = [&](int tile_id, int& bb, int& r0, int& ln, int64_t& t0) {
-        if (!VARLEN) {
-            const int tiles = (p.L + BM - 1) / BM;
-            bb = tile_id / tiles;
-            r0 = (tile_id - bb * tiles) * BM;
-            ln = !p.seqlens ? p.L : bb < 64 ? lds_int(&sm.seq_n[bb]) : min(max(p.seqlens[bb], 0), p.L);
-            t0 = 0;
-            return true;
-        }
-        int t = tile_id;
-        for (int b0 = 0; b0 < p.B; b0 += 64) {
-            const int bx = b0 + l;
-            int s0 = 0, n = 0;
-            if (bx < p.B) {
-                s0 = p.cu_seqlens[bx];
-                const int e = p.cu_seqlens[bx + 1];
-                n = e - s0;
-                if (s0 < 0 || n < 0 || e > p.total) n = 0;   // malformed entry: no tiles
-                n = min(n, p.L);
-            }
-            const int nt = (n + BM - 1) / BM;
-            int incl = nt;                                   // inclusive prefix sum over the wave
-#pragma unroll
-            for (int d = 1; d < 64; d <<= 1) {
-                const int up = __shfl_up(incl, d);
-                if (l >= d) incl += up;
-            }
-            const int chunk_tiles = __builtin_amdgcn_readlane(incl, 63);
-            if (t < chunk_tiles) {
-                const unsigned long long owners = __builtin_amdgcn_ballot_w64(incl > t);
-                const int ln_ = __builtin_amdgcn_readfirstlane(__builtin_ctzll(owners));
-                const int before = __builtin_amdgcn_readlane(incl, ln_) - __builtin_amdgcn_readlane(nt, ln_);
-                bb = b0 + ln_;
-                r0 = (t - before) * BM;
-                ln = __builtin_amdgcn_readlane(n, ln_);
-                t0 = __builtin_amdgcn_readlane(s0, ln_);
-                return true;
-            }
-            t -= chunk_tiles;
-        }
-        return false;
+        const int tiles = (p.L + BM - 1) / BM;
+        bb = tile_id / tiles;
+        r0 = (tile_id - bb * tiles) * BM;
+        ln = !p.seqlens ? p.L : bb < 64 ? lds_int(&sm.seq_n[bb]) : min(max(p.seqlens[bb], 0), p.L);
+        t0 = 0;
+        return true;
     };
     constexpr int TEAM = TEAM_MAX;
     // deal state of this wave: cost per member, then [+0] cost coordinate of the next tile of the list, [+1] end of
