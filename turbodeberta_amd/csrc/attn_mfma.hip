@@ -189,11 +189,13 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         return int64_t((uint64_t(uint32_t(hi)) << 32) | uint32_t(lo));
     };
     auto tiles_of = [](int n) { return (n + BM - 1) / BM; };
-    auto cost_of = [](int n) { return int64_t(8 * ((n + BN - 1) / BN) + 13); };
+    auto cost_of = [](int n) { return int64_t(8 * ((n + BN - 1) / BN) + 24); };
     // Packed launches (at most 64 sequences: the launcher splits larger batches) use a cost-balanced walk instead of
-    // the strided one of the fixed layout: tiles differ in length by up to 8x, so a TEAM of workgroups takes a CONTIGUOUS range of the tile list (heads outermost, then
-    // sequences, then the query tiles of a sequence) whose summed cost is its share of the total.  The cost of a tile
-    // is 8 * (its key steps) + 13, in eighths of a key step (13: what opening a tile costs).  Every wave derives the
+    // the strided one of the fixed layout: tiles differ in length by up to 8x, so a TEAM of workgroups takes a
+    // CONTIGUOUS range of the tile list (heads outermost, then sequences, then the query tiles of a sequence) whose
+    // summed cost is its share of the total.  The cost of a tile is 8 * (its key steps) + 24, in eighths of a key
+    // step (24: what a tile costs beside its steps; measured, the launch time is flat between 24 and 32 and 2.5 %
+    // higher at 13 or 40).  Every wave derives the
     // same ranges from the sequence boundaries; a tile belongs to the team whose cost interval holds the tile's
     // start coordinate.  A team is TEAM workgroups that sit on one XCD (block ids go round-robin over the 8 XCDs);
     // inside a team the tiles are dealt in list order, each to the member with the least cost so far -- what a
