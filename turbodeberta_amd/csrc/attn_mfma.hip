@@ -219,15 +219,17 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         } else if (p.seqlens) {
             n = min(max(p.seqlens[min(l, p.B - 1)], 0), p.L);
         }
-        int64_t pre = tiles_of(n) * cost_of(n);                          // inclusive prefix sum over the wave
-#pragma unroll
-        for (int d = 1; d < 64; d <<= 1) {
-            const int64_t up = __shfl_up(pre, d);
-            if (l >= d) pre += up;
-        }
         sm.seq_n[l] = n;
-        sm.seq_lo[l] = lo;
-        sm.seq_pre[l] = pre;
+        if (VARLEN) {                     // (the fixed layout's walk needs the lengths only)
+            int64_t pre = tiles_of(n) * cost_of(n);                      // inclusive prefix sum over the wave
+#pragma unroll
+            for (int d = 1; d < 64; d <<= 1) {
+                const int64_t up = __shfl_up(pre, d);
+                if (l >= d) pre += up;
+            }
+            sm.seq_lo[l] = lo;
+            sm.seq_pre[l] = pre;
+        }
     }
     // fixed layout: tile_id -> (sequence, first row, valid length); same map as tdb_locate_tile
     auto locate = [&](int tile_id, int& bb, int& r0, int& ln, int64_t& t0) {
