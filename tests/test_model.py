@@ -86,6 +86,63 @@ def test_pack_unpack_round_trip():
     assert torch.equal(q, packed) and pk is None and torch.equal(cq, cu) and mq == 5
 
 
+def test_mask_shapes_accepted_and_rejected():
+    from turbodeberta_amd.model import _mask_info
+    m2 = torch.tensor([[1, 1, 1, 0, 0], [1, 1, 1, 1, 1], [1, 0, 0, 0, 0]])
+    outer = m2[:, :, None] * m2[:, None, :]
+    row = m2[:, None, None, :]                                    # the "extended" key mask [B, 1, 1, L]
+    accepted = (m2, outer, outer[:, None], outer[:, None].expand(3, 4, 5, 5), row, row.expand(3, 4, 1, 5), m2[:, None, :])
+    for m in accepted:
+        info = _mask_info(m.clone())
+        assert info.lengths.tolist() == [3, 5, 1] and info.total == 9, tuple(m.shape)
+        assert torch.equal(padding.key_padding_mask(m), m2)
+    # a broadcast key mask must not be read through a "diagonal" of its single row
+    assert _mask_info(torch.ones(2, 1, 1, 7)).lengths.tolist() == [7, 7]
+    # shapes with no token axis to read
+    for bad in (torch.ones(3, 1, 2, 5), torch.ones(3, 4, 5), torch.ones(3, 5, 4)):
+        with pytest.raises(ValueError, match="last two dimensions"):
+            _mask_info(bad)
+    # heads that differ: only head 0 would have been looked at
+    per_head = outer[:, None].repeat(1, 2, 1, 1)
+    per_head[1, 1, 4, 4] = 0
+    with pytest.raises(ValueError, match="right padded"):
+        _mask_info(per_head)
+    per_head_row = row.repeat(1, 2, 1, 1)
+    per_head_row[0, 1, 0, 2] = 0
+    with pytest.raises(ValueError, match="right padded"):
+        _mask_info(per_head_row)
+    # holes, left padding, a square mask that is not an outer product
+    for bad in (torch.tensor([[1, 0, 1, 0]]), torch.tensor([[0, 1, 1, 1]])):
+        with pytest.raises(ValueError, match="right padded"):
+            _mask_info(bad)
+    causal = torch.tril(torch.ones(1, 4, 4, dtype=torch.long))
+    with pytest.raises(ValueError, match="right padded"):
+        _mask_info(causal)
+
+
+def test_model_passes_the_hidden_state_wish_as_an_argument():
+    """The model tells the encoder per call (not through module state) whether the layers' outputs are wanted."""
+    m = FlashDebertaV2Model(_tiny()).eval()
+    seen = []
+
+    class Stop(Exception):
+        pass
+
+    def spy(hidden_states, attention_mask, **kw):
+        seen.append(kw.get("intermediate_states", True))
+        raise Stop
+
+    m.encoder.forward = spy
+    ids, mask = (torch.from_numpy(a) for a in tiny_model_inputs())
+    for wish, expected in ((None, False), (False, False), (True, True)):
+        with pytest.raises(Stop):
+            m(input_ids=ids, attention_mask=mask, output_hidden_states=wish)
+        assert seen[-1] is expected
+    assert not any(k.startswith("_tdb_all") for k in vars(m.encoder))
+    with pytest.raises(ValueError, match="exactly one"):
+        m(input_ids=ids, inputs_embeds=torch.zeros(2, 3, 4))
+
+
 # ------------------------------------------------------------------------------------- GPU
 
 @pytest.mark.gpu

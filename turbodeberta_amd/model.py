@@ -81,7 +81,8 @@ def _mask_info(attention_mask):
     """Valid lengths of a batch whose mask is **right padded** (valid tokens first), verified: the kernels take
     per-sequence lengths, so a mask with holes or left padding cannot be expressed and raises ``ValueError`` instead
     of attending to the wrong tokens.  A 3-D / 4-D mask must be the outer product ``m_i * m_j`` Hugging Face's
-    encoder builds (modeling_deberta_v2.py:601-608).  The check costs one host synchronisation per mask object;
+    encoder builds (modeling_deberta_v2.py:601-608), or one row ``[.., 1, L]`` that broadcasts over the queries, and the
+    same for every head; other shapes raise ``ValueError`` in ``key_padding_mask``.  The check costs one host synchronisation per mask object;
     the result is attached to the tensor, so the layers of an encoder, which all receive the same mask object
     (modeling_deberta_v2.py:651-660), share it.  (A mask without a modification counter -- an inference tensor --
     is trusted not to be modified in place between calls.)"""
@@ -93,14 +94,17 @@ def _mask_info(attention_mask):
     L = valid.shape[-1]
     lengths = valid.sum(dim=-1, dtype=torch.int32)
     ok = (valid == (torch.arange(L, device=valid.device)[None, :] < lengths[:, None])).all()
-    if attention_mask.dim() > 2:
+    if attention_mask.dim() == 4 and attention_mask.shape[1] > 1:
+        ok = ok & ((attention_mask != 0) == (attention_mask[:, :1] != 0)).all()      # one length per sequence: no per-head masks
+    if attention_mask.dim() > 2 and attention_mask.shape[-2] == L and L > 1:
         full = attention_mask if attention_mask.dim() == 3 else attention_mask[:, 0]
         ok = ok & ((full != 0) == (valid[:, :, None] & valid[:, None, :])).all()
     ok_host, total = torch.stack([ok.to(torch.int64), lengths.sum(dtype=torch.int64)]).tolist()   # the one synchronisation
     if not ok_host:
         raise ValueError("attention_mask must be right padded (valid tokens first, no holes) and, if 3-D or 4-D, the "
-                         "outer product of a key-padding mask with itself: the fused attention takes per-sequence "
-                         "lengths.  Use the eager Hugging Face modules for other masks.")
+                         "outer product of a key-padding mask with itself (or one broadcast row of it), equal for all "
+                         "heads: the fused attention takes per-sequence lengths.  Use the eager Hugging Face modules for "
+                         "other masks.")
     info = _MaskInfo(lengths, int(total))
     try:
         attention_mask._tdb_info = (version, info)
@@ -268,7 +272,6 @@ class FlashDebertaV2Encoder(DebertaV2Encoder):
     ``pack_sequences = False`` switches the packed path off."""
 
     pack_sequences = True
-    _tdb_all_hidden = True      # cleared by FlashDebertaV2Model when the caller did not ask for every layer's output
 
     def __init__(self, config):
         super().__init__(config)
@@ -295,7 +298,10 @@ class FlashDebertaV2Encoder(DebertaV2Encoder):
         return cached[1]
 
     def forward(self, hidden_states, attention_mask, output_hidden_states=True, output_attentions=False,
-                query_states=None, relative_pos=None, return_dict=True):
+                query_states=None, relative_pos=None, return_dict=True, intermediate_states=True):
+        """As the parent (modeling_deberta_v2.py:634-695).  ``intermediate_states=False`` (an argument of this class
+        only) says that of the hidden states the caller reads just the first and the last: the packed path then
+        leaves the layers in between out of the returned tuple instead of scattering each back to ``[B, L, hidden]``."""
         fused = (not output_attentions and torch.is_tensor(hidden_states)
                  and all(isinstance(l.attention.self, FlashDisentangledSelfAttention) for l in self.layer))
         packable = (fused and self.pack_sequences and not self.training and not torch.is_grad_enabled()
@@ -312,7 +318,7 @@ class FlashDebertaV2Encoder(DebertaV2Encoder):
             return super().forward(hidden_states, attention_mask, output_hidden_states, output_attentions,
                                    query_states, relative_pos, return_dict)
 
-        keep_all = output_hidden_states and self._tdb_all_hidden
+        keep_all = output_hidden_states and intermediate_states
         padded = lambda t: pad_input(t, indices, B, L)
         all_hidden_states = (hidden_states,) if output_hidden_states else None
         rel_embeddings = self.get_rel_embedding()
@@ -342,18 +348,37 @@ class FlashDebertaV2Model(DebertaV2Model):
 
     def forward(self, input_ids=None, attention_mask=None, token_type_ids=None, position_ids=None,
                 inputs_embeds=None, output_attentions=None, output_hidden_states=None, return_dict=None, **kwargs):
-        # The parent always asks the encoder for every layer's output and then uses the last one
-        # (modeling_deberta_v2.py:760-768); tell the packed encoder whether the caller wants the others too,
-        # so that it does not scatter 24 intermediate results back to [B, L, hidden] for nothing.
-        wanted = output_hidden_states if output_hidden_states is not None else self.config.output_hidden_states
-        self.encoder._tdb_all_hidden = bool(wanted) or self.z_steps > 1
-        try:
+        """As the parent (modeling_deberta_v2.py:711-793), which always asks the encoder for every layer's output and
+        then uses the last one (modeling_deberta_v2.py:760-768).  When the caller did not ask for the hidden states
+        (and no ``z_steps`` pass needs the last but one), the encoder is told so through its ``intermediate_states``
+        argument, so that the packed path does not scatter every layer's result back to ``[B, L, hidden]`` for
+        nothing.  Nothing is stored on the modules: concurrent calls on one model do not see each other's flags."""
+        cfg = self.config
+        want_hidden = output_hidden_states if output_hidden_states is not None else cfg.output_hidden_states
+        if want_hidden or self.z_steps > 1 or kwargs:
             return super().forward(input_ids=input_ids, attention_mask=attention_mask, token_type_ids=token_type_ids,
                                    position_ids=position_ids, inputs_embeds=inputs_embeds,
                                    output_attentions=output_attentions, output_hidden_states=output_hidden_states,
                                    return_dict=return_dict, **kwargs)
-        finally:
-            self.encoder._tdb_all_hidden = True
+        output_attentions = output_attentions if output_attentions is not None else cfg.output_attentions
+        return_dict = return_dict if return_dict is not None else cfg.return_dict
+        if (input_ids is None) == (inputs_embeds is None):
+            raise ValueError("You have to specify exactly one of input_ids and inputs_embeds")
+        given = input_ids if input_ids is not None else inputs_embeds[..., 0]
+        if input_ids is not None:
+            self.warn_if_padding_and_no_attention_mask(input_ids, attention_mask)
+        if attention_mask is None:
+            attention_mask = torch.ones(given.shape, device=given.device)
+        if token_type_ids is None:
+            token_type_ids = torch.zeros(given.shape, dtype=torch.long, device=given.device)
+        embedded = self.embeddings(input_ids=input_ids, token_type_ids=token_type_ids, position_ids=position_ids,
+                                   mask=attention_mask, inputs_embeds=inputs_embeds)
+        encoded = self.encoder(embedded, attention_mask, output_hidden_states=True, output_attentions=output_attentions,
+                               return_dict=return_dict, intermediate_states=False)
+        sequence_output = encoded[1][-1]
+        if not return_dict:
+            return (sequence_output,) + tuple(encoded[2:])
+        return BaseModelOutput(last_hidden_state=sequence_output, hidden_states=None, attentions=encoded.attentions)
 
 
 class _FusedHead:

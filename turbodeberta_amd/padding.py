@@ -12,15 +12,24 @@ import torch.nn.functional as F
 def key_padding_mask(attention_mask: torch.Tensor) -> torch.Tensor:
     """``[B, L]`` validity of every token from the masks Hugging Face passes around: a 2-D mask is
     returned as is; the encoder's ``[B, 1, L, L]`` (``m_i * m_j``, modeling_deberta_v2.py:601-608) or a
-    ``[B, L, L]`` mask is reduced through its diagonal ``m_i * m_i`` -- a view, no reduction kernel.
-    (The reference assumes 2-D, padding.py:79-83, and breaks on the encoder's 4-D mask.)"""
+    ``[B, L, L]`` mask is reduced through its diagonal ``m_i * m_i`` -- a view, no reduction kernel; a
+    mask with one query row that broadcasts over the queries (``[B, 1, L]``, ``[B, 1, 1, L]``, the
+    "extended" key mask of other Hugging Face models) is that row.  Of a mask with several heads, head 0 is
+    taken.  Any other shape raises ``ValueError``: a mask whose last two dimensions differ has no diagonal to
+    read the tokens from.  (The reference assumes 2-D, padding.py:79-83, and breaks on the encoder's 4-D mask.)"""
     if attention_mask.dim() == 2:
         return attention_mask
     if attention_mask.dim() == 4:
         attention_mask = attention_mask[:, 0]
     if attention_mask.dim() != 3:
         raise ValueError(f"attention_mask must have 2, 3 or 4 dims, got {attention_mask.dim()}")
-    return torch.diagonal(attention_mask, dim1=-2, dim2=-1)
+    rows, cols = attention_mask.shape[-2:]
+    if rows == cols:
+        return torch.diagonal(attention_mask, dim1=-2, dim2=-1)
+    if rows == 1:
+        return attention_mask[:, 0]
+    raise ValueError(f"attention_mask of shape {tuple(attention_mask.shape)}: the last two dimensions must be "
+                     f"[L, L] or [1, L]")
 
 
 def sequence_lengths(attention_mask: torch.Tensor) -> torch.Tensor:
