@@ -20,7 +20,7 @@
 extern "C" {
 #endif
 
-#define TDB_ABI_VERSION 1
+#define TDB_ABI_VERSION 2
 
 /* status codes */
 #define TDB_OK                 0
@@ -153,6 +153,17 @@ int tdb_delta_table(int32_t* out, int32_t max_len, int32_t position_buckets, int
  * synchronisation; on the device a malformed entry makes that sequence's tiles exit early.)
  */
 int tdb_check_cu_seqlens(const int32_t* cu_seqlens_host, int32_t batch, int32_t total_tokens, int32_t max_seqlen);
+
+/*
+ * Process-wide cap on the persistent workgroups (one per compute unit) that a matrix-core launch
+ * starts: `workgroups` is rounded down to a multiple of 8 (one per XCD at least: minimum 8);
+ * 0 or a negative value lifts the cap (default: every compute unit of the device).  For callers
+ * that share the GPU with other streams, and for tests of the packed tile deal at other grid
+ * sizes than this device's.  Returns the cap now in force (0 = none).  No counterpart in the
+ * reference, whose launch grid is one program per tile (ops/flash_attention.py:360,
+ * ops/flash_attention_varlen.py:328).
+ */
+int tdb_set_workgroup_limit(int workgroups);
 
 #ifdef __cplusplus
 }

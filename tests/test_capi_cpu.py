@@ -26,6 +26,14 @@ def test_library_exports_every_declared_symbol():
     assert int(m.group(1)) == _lib.ABI_VERSION
 
 
+def test_workgroup_limit_rounding():
+    try:
+        assert [_lib.set_workgroup_limit(n) for n in (1, 8, 15, 24, 250, 4096)] == [8, 8, 8, 24, 248, 4096]
+        assert _lib.set_workgroup_limit(-3) == 0
+    finally:
+        assert _lib.set_workgroup_limit(0) == 0
+
+
 def test_struct_layout_matches_header_field_order():
     header = open(os.path.join(ROOT, "include", "tdb_attn.h")).read()
     for cname, cls in (("tdb_pos_args", _lib.PosArgs), ("tdb_fixed_args", _lib.FixedArgs), ("tdb_varlen_args", _lib.VarlenArgs)):

@@ -120,6 +120,22 @@ def test_mask_shapes_accepted_and_rejected():
         _mask_info(causal)
 
 
+def test_declared_masks_are_not_inspected():
+    from turbodeberta_amd.model import _mask_info, declare_right_padded
+    holes = torch.tensor([[1, 0, 1, 0], [1, 1, 1, 1]])                 # would be refused if it were looked at
+    lengths = torch.tensor([2, 4], dtype=torch.int32)
+    assert declare_right_padded(holes, lengths) is holes
+    info = _mask_info(holes)
+    assert info.lengths is lengths and info.total is None
+    assert _mask_info(declare_right_padded(holes, lengths, total=6)).total == 6
+    holes[1, 1] = 0                                                    # an in-place edit voids the declaration
+    with pytest.raises(ValueError, match="right padded"):
+        _mask_info(holes)
+    for bad in (lengths.long(), lengths[:1], lengths[None]):
+        with pytest.raises(ValueError, match="lengths"):
+            declare_right_padded(holes, bad)
+
+
 def test_model_passes_the_hidden_state_wish_as_an_argument():
     """The model tells the encoder per call (not through module state) whether the layers' outputs are wanted."""
     m = FlashDebertaV2Model(_tiny()).eval()
@@ -160,6 +176,29 @@ def test_tiny_model_matches_hf_golden(golden_dir):
     valid = torch.from_numpy(mask).bool()
     rel = (out[valid] - gold[valid]).abs().max() / gold[valid].abs().max()
     assert rel <= 1e-4, rel
+
+
+@pytest.mark.gpu
+def test_declared_mask_gives_the_same_result_without_packing():
+    """A mask declared right padded (no inspection, no host synchronisation) without a token count keeps the padded
+    layout; with the count the encoder packs.  Both must reproduce the inspected-mask result on the valid tokens."""
+    from turbodeberta_amd.model import declare_right_padded
+    model = FlashDebertaV2Model(_tiny()).eval()
+    fill_params(model)
+    model = model.to("cuda:0")
+    ids, mask = tiny_model_inputs()
+    ids, mask = torch.from_numpy(ids).cuda(), torch.from_numpy(mask).cuda()
+    valid = mask.bool()
+    lengths = mask.sum(-1, dtype=torch.int32)
+    with torch.no_grad():
+        want = model(input_ids=ids, attention_mask=mask.clone()).last_hidden_state
+        print("[case] declared mask, padded layout", flush=True)
+        padded = model(input_ids=ids, attention_mask=declare_right_padded(mask.clone(), lengths)).last_hidden_state
+        print("[case] declared mask, packed layout", flush=True)
+        packed = model(input_ids=ids, attention_mask=declare_right_padded(mask.clone(), lengths, int(lengths.sum()))
+                       ).last_hidden_state
+    assert torch.equal(packed[valid], want[valid])
+    assert torch.allclose(padded[valid], want[valid], atol=2e-5, rtol=0)
 
 
 @pytest.mark.gpu

@@ -262,6 +262,40 @@ def test_bf16_varlen_more_than_64_sequences(force_generic):
             assert torch.equal(part, out[lo:hi]), f"sequences {first}..{first + 49}"
 
 
+def test_packed_tile_deal_at_other_grid_sizes():
+    """The packed launch deals its tiles to the persistent workgroups inside the kernel.  Grids of 8, 24 and 40
+    workgroups (24 and 40 are not multiples of 16: teams of one) and the full device must all produce every tile:
+    the output is zero-filled first, so a tile that nobody took would stay zero, and each result must equal the
+    full-grid one bit for bit (a tile's arithmetic does not depend on who computes it)."""
+    from turbodeberta_amd import _lib
+    H, D, buckets, max_rel = 16, 64, 256, 512
+    rs = np.random.RandomState(7)
+    lengths = [int(x) for x in rs.randint(1, 260, size=64)]
+    for i in (0, 5, 31, 63):
+        lengths[i] = 0
+    lengths[17] = 300
+    inp = make_inputs(21, len(lengths), H, max(lengths), D, buckets, max_rel, dtype=torch.bfloat16)
+    packed, cu = pack(inp, lengths)
+    f = lambda t: t.float()
+    ref = O.attention_varlen(f(packed["q"]), f(packed["k"]), f(packed["v"]), f(inp["pk"]), f(inp["pq"]), cu,
+                             position_buckets=buckets, max_relative_positions=max_rel)
+    dev = {k: packed[k].to(DEV) for k in ("q", "k", "v")}
+    run = lambda: flash_attention_with_disentangled_varlen(
+        dev["q"], dev["k"], dev["v"], None, None, cu.to(DEV), cu.to(DEV), max(lengths), max(lengths), False,
+        1 / math.sqrt(3 * D), buckets, max_rel, pos_key_layer=inp["pk"].to(DEV), pos_query_layer=inp["pq"].to(DEV))
+    try:
+        print("[case] packed deal, full grid", flush=True)
+        assert _lib.set_workgroup_limit(0) == 0
+        full = run()
+        assert_close_bf16(full.cpu(), ref, "packed deal, full grid")
+        for grid in (8, 24, 40, 250):
+            print(f"[case] packed deal, at most {grid} workgroups", flush=True)
+            assert _lib.set_workgroup_limit(grid) == grid // 8 * 8
+            assert torch.equal(run(), full), f"grid {grid}"
+    finally:
+        _lib.set_workgroup_limit(0)
+
+
 @pytest.mark.parametrize("force_generic", [False, True])
 @pytest.mark.parametrize("B,H,L,buckets,max_rel,lengths", [
     (2, 4, 512, 256, 512, (512, 389)),

@@ -15,7 +15,7 @@ LIB_PATH = os.path.join(PKG, "libtdb_attn.so")
 
 TDB_F32, TDB_BF16, TDB_F16 = 0, 1, 2
 TDB_FLAG_FORCE_GENERIC = 1
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 ERROR_NAMES = {
     -1: "TDB_ERR_NULL", -2: "TDB_ERR_DTYPE", -3: "TDB_ERR_SHAPE", -4: "TDB_ERR_STRIDE", -5: "TDB_ERR_ALIGN",
@@ -26,7 +26,7 @@ ERROR_NAMES = {
 _VALUE_ERRORS = {-1, -2, -3, -4, -5, -6, -7, -8, -9}
 
 EXPORTS = ("tdb_version", "tdb_last_error", "tdb_attn_fwd_fixed", "tdb_attn_fwd_varlen", "tdb_bucket_table",
-           "tdb_delta_table", "tdb_check_cu_seqlens")
+           "tdb_delta_table", "tdb_check_cu_seqlens", "tdb_set_workgroup_limit")
 
 
 class PosArgs(C.Structure):
@@ -99,6 +99,8 @@ def load() -> C.CDLL:
             fn.restype = C.c_int
         lib.tdb_check_cu_seqlens.argtypes = [C.c_void_p, C.c_int32, C.c_int32, C.c_int32]
         lib.tdb_check_cu_seqlens.restype = C.c_int
+        lib.tdb_set_workgroup_limit.argtypes = [C.c_int]
+        lib.tdb_set_workgroup_limit.restype = C.c_int
         if lib.tdb_version() != ABI_VERSION:
             raise RuntimeError(f"libtdb_attn.so has ABI {lib.tdb_version()}, this package expects {ABI_VERSION}")
         _lib = lib
@@ -128,3 +130,9 @@ def delta_table(max_len: int, position_buckets: int, max_position: int) -> np.nd
 def check_cu_seqlens(cu_host: np.ndarray, total_tokens: int, max_seqlen: int) -> None:
     cu = np.ascontiguousarray(cu_host, dtype=np.int32)
     check(load().tdb_check_cu_seqlens(cu.ctypes.data, len(cu) - 1, total_tokens, max_seqlen))
+
+
+def set_workgroup_limit(workgroups: int) -> int:
+    """Cap the persistent workgroups (one per compute unit) of the matrix-core launches of this process;
+    0 lifts the cap.  Returns the cap in force (a multiple of 8)."""
+    return int(load().tdb_set_workgroup_limit(int(workgroups)))

@@ -33,6 +33,7 @@
 //         P'[j][i - j - B_s], which becomes the initial value of the S^T accumulator.
 // Together: S[i,j] = Q_i.K_j + Q_i.K_r[delta(i-j)] + K_j.Q_r[delta(i-j)], the Hugging Face eager
 // definition (modeling_deberta_v2.py:317-324, :337-343).
+#include <atomic>
 #include <mutex>
 #include <type_traits>
 #include <utility>
@@ -1206,8 +1207,15 @@ constexpr int kInstances = 32;
 std::mutex g_dev_mutex;
 int g_cus[kMaxDevices] = {0};
 bool g_attr_set[kMaxDevices][kInstances] = {{false}};
+std::atomic<int> g_workgroup_limit{0};       // cap on the persistent workgroups of a launch (multiple of 8), 0 = none
 
 }  // namespace
+
+int tdb_mfma_set_workgroup_limit(int workgroups) {
+    const int cap = workgroups <= 0 ? 0 : workgroups < 8 ? 8 : workgroups / 8 * 8;
+    g_workgroup_limit.store(cap, std::memory_order_relaxed);
+    return cap;
+}
 
 hipError_t tdb_launch_mfma(const TdbKernelParams& whole, int dtype, hipStream_t stream) {
     // Packed batches of more than 64 sequences go out as several launches of at most 64 (even parts): the kernel
@@ -1273,6 +1281,8 @@ hipError_t tdb_launch_mfma(const TdbKernelParams& whole, int dtype, hipStream_t 
     }
     // Persistent workgroups, one per CU: fixed layout with a strided deal (tiles cost about the same), packed
     // batches with a cost-balanced deal computed in the kernel.
+    const int limit = g_workgroup_limit.load(std::memory_order_relaxed);
+    if (limit > 0 && limit < cus) cus = limit;
     const int persistent = nblocks < cus ? nblocks : cus;
     void* args[] = {const_cast<TdbKernelParams*>(&p), const_cast<int*>(&nblocks)};
     return hipLaunchKernel(fn, dim3(unsigned(persistent)), dim3(NTHREADS), args, smem, stream);

@@ -166,6 +166,8 @@ int tdb_check_cu_seqlens(const int32_t* cu, int32_t batch, int32_t total_tokens,
     return TDB_OK;
 }
 
+int tdb_set_workgroup_limit(int workgroups) { return tdb_mfma_set_workgroup_limit(workgroups); }
+
 int tdb_attn_fwd_fixed(const tdb_fixed_args* a, void* stream) {
     if (!a) return fail(TDB_ERR_NULL, "args is NULL");
     int rc = check_common(a->dtype, a->batch, a->heads, a->head_dim, a->seqlen, a->causal, a->q, a->k, a->v, a->o);

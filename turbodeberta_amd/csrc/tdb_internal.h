@@ -42,6 +42,8 @@ bool tdb_mfma_supported(const TdbKernelParams& p, int dtype);
 // launchers; return hipError_t of the launch
 hipError_t tdb_launch_generic(const TdbKernelParams& p, int dtype, hipStream_t stream);
 hipError_t tdb_launch_mfma(const TdbKernelParams& p, int dtype, hipStream_t stream);
+// Cap on the persistent workgroups of a launch (multiple of 8, 0 = none); returns the cap in force.
+int tdb_mfma_set_workgroup_limit(int workgroups);
 
 // Maps blockIdx.x to (sequence, first row of the tile, valid length).  Returns false when the
 // block has no tile (packed launches are sized by an upper bound on the tile count).  Must be

@@ -70,7 +70,7 @@ def _version_of(t):
 
 class _MaskInfo:
     """What the fused paths need to know about an attention mask: ``lengths`` int32 ``[B]`` on the device and
-    ``total``, the number of valid tokens (a host int)."""
+    ``total``, the number of valid tokens (a host int; ``None`` when the caller declared the lengths without it)."""
     __slots__ = ("lengths", "total")
 
     def __init__(self, lengths, total):
@@ -111,6 +111,22 @@ def _mask_info(attention_mask):
     except AttributeError:      # tensor subclasses without a __dict__
         pass
     return info
+
+
+def declare_right_padded(attention_mask, lengths, total=None):
+    """Opt out of the mask inspection: the caller vouches that ``attention_mask`` is right padded with ``lengths``
+    (int32 ``[B]`` on the mask's device) valid tokens per sequence.  The facts are attached to the mask tensor the way
+    ``_mask_info`` caches its own findings, so every fused module that receives this mask object uses them and none
+    synchronises with the host: a forward on such a mask can be captured into a HIP graph.  ``total`` (a host int, the
+    sum of the lengths) additionally lets the encoder pack the batch; without it the encoder keeps the padded layout,
+    because the packed token count sizes host-side allocations.  Nothing is verified: wrong lengths give wrong
+    attention.  Returns the mask."""
+    if lengths.dtype != torch.int32 or lengths.dim() != 1 or lengths.shape[0] != attention_mask.shape[0]:
+        raise ValueError("lengths must be an int32 tensor with one entry per sequence of the mask")
+    if lengths.device != attention_mask.device:
+        raise ValueError("lengths must live on the mask's device")
+    attention_mask._tdb_info = (_version_of(attention_mask), _MaskInfo(lengths, None if total is None else int(total)))
+    return attention_mask
 
 
 def _packing_of(info, batch, seqlen, device):
@@ -309,7 +325,7 @@ class FlashDebertaV2Encoder(DebertaV2Encoder):
         if packable:
             B, L, _ = hidden_states.shape
             info = _mask_info(attention_mask)                                # the one host synchronisation
-            packable = info.total < B * L
+            packable = info.total is not None and info.total < B * L      # (no total: declared by the caller)
             if packable:
                 indices, cu_seqlens = _packing_of(info, B, L, hidden_states.device)
         if not packable:
