@@ -44,32 +44,57 @@ PEAK_HBM_GBS = 8000.0
 METRIC = "attn TFLOP/s + tokens/s, DeBERTa-v3-base b32xL512 bf16, fixed and varlen"
 PEAK_FP32_VALU_TFLOPS = 157.3   # MI355X vector fp32, AMD public spec (what the generic kernel is priced against)
 # HBM bytes per launch are not measured by this script: they come from `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE`
-# runs of it, each counter scaled by what it reads for a plain 512 MiB device copy.  The figures, the commands and the
-# commit they were taken at are recorded in the files named here; `roofline.traffic` repeats them with that source.
+# runs of it, each counter scaled by what it reads for a plain 512 MiB device copy.  The figures, the commands, the
+# commit and a digest of the kernel source they were taken at are recorded in the files named here; `roofline.traffic`
+# repeats them with that source, and `roofline.traffic_stale` is true when the kernel source has changed since.
 RECORDED_TRAFFIC = {
-    "fixed": ("profiles/attn_mfma_kernel_fixed_b32xL512.md", None),
-    "varlen": ("profiles/attn_mfma_kernel_varlen_64seq.md", None),
+    "fixed": "profiles/attn_mfma_kernel_fixed_b32xL512.md",
+    "varlen": "profiles/attn_mfma_kernel_varlen_64seq.md",
+    "long": "profiles/attn_mfma_kernel_long_b4xL4096.md",
+    "long_varlen": "profiles/attn_mfma_kernel_long_b4xL4096.md",
 }
+KERNEL_SOURCES = ("turbodeberta_amd/csrc/attn_mfma.hip", "turbodeberta_amd/csrc/tdb_internal.h")
+
+
+def kernel_source_digest():
+    """First 16 hex digits of the SHA-256 over the matrix-core kernel's source files, in the order of KERNEL_SOURCES:
+    what a profile summary records as `kernel_source_sha256:` when its counters are taken."""
+    import hashlib
+    h = hashlib.sha256()
+    try:
+        for rel in KERNEL_SOURCES:
+            h.update(open(os.path.join(ROOT, rel), "rb").read())
+    except OSError:
+        return None
+    return h.hexdigest()[:16]
 
 
 def recorded_traffic(name):
-    """(bytes, source) from the profile summary of a workload: the line `traffic_bytes_per_launch: <number>` and the
-    line `commit: <hash>` of the file; (None, None) when the file or the line is missing."""
-    path = RECORDED_TRAFFIC.get(name, (None, None))[0]
+    """(bytes, source, stale) from the profile summary of a workload: the line `traffic_bytes_per_launch: <number>`
+    (`traffic_bytes_per_launch[<name>]:` when one file covers several workloads), the line `commit: <hash>` and the
+    line `kernel_source_sha256: <digest>` of the file.  `stale` says that the kernel source has changed since the
+    counters were read (or that the summary does not say what it was read from); (None, None, None) when the file or
+    the line is missing."""
+    path = RECORDED_TRAFFIC.get(name)
     if path is None:
-        return None, None
+        return None, None, None
     try:
         text = open(os.path.join(ROOT, path)).read()
     except OSError:
-        return None, None
-    val = commit = None
+        return None, None, None
+    val = commit = digest = None
     for line in text.splitlines():
-        if line.startswith("traffic_bytes_per_launch:"):
-            val = float(line.split(":", 1)[1])
+        for key in ("traffic_bytes_per_launch:", f"traffic_bytes_per_launch[{name}]:"):
+            if line.startswith(key):
+                val = float(line.split(":", 1)[1])
         if line.startswith("commit:"):
             commit = line.split(":", 1)[1].strip()
-    return val, (f"{path} (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, calibrated on a 512 MiB copy; commit {commit})"
-                 if val is not None else None)
+        if line.startswith("kernel_source_sha256:"):
+            digest = line.split(":", 1)[1].strip()
+    if val is None:
+        return None, None, None
+    source = f"{path} (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, calibrated on a 512 MiB copy; commit {commit})"
+    return val, source, digest is None or digest != kernel_source_digest()
 
 
 def flops_of(lengths, heads=H) -> float:
@@ -364,13 +389,14 @@ def main():
         spent_prewarm.append(spent)
         fl = flops_of(lengths)
         ach = fl / (mean_ms * 1e-3) / 1e12
-        traffic, traffic_source = recorded_traffic(name)
+        traffic, traffic_source, traffic_stale = recorded_traffic(name)
         return {
             "value": round(fl / (wall_ms * 1e-3) / 1e12, 2), "ms_per_step": round(wall_ms, 4), "steps": steps,
             "tokens_per_s": round(float(lengths.sum()) / (wall_ms * 1e-3), 1),
             "core_tflops": round(H * sum(4.0 * int(l) ** 2 * D for l in lengths) / (wall_ms * 1e-3) / 1e12, 2),
             "roofline": {"bound": bound, "achieved": round(ach, 2), "peak": peak, "unit": "TFLOP/s",
-                         "frac": round(ach / peak, 4), "traffic": traffic, "traffic_source": traffic_source, "kernel": kernel,
+                         "frac": round(ach / peak, 4), "traffic": traffic, "traffic_source": traffic_source, "traffic_stale": traffic_stale,
+                         "kernel": kernel,
                          "kernel_ms_mean": round(mean_ms, 4), "kernel_ms_pair_median": round(med_ms, 4),
                          "kernel_ms_pair_min": round(min_ms, 4), "algorithmic_gflop": round(fl / 1e9, 3), "algorithmic_bytes": algorithmic_bytes(lengths),
                          "hbm_gbs_algorithmic": round(algorithmic_bytes(lengths) / (mean_ms * 1e-3) / 1e9, 1)},

@@ -519,6 +519,14 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         // ================================================= position waves ==========================================
         const int stid = tid - 256;
         const int srow = stid >> 3, sch = stid & 7;          // this thread stages rows srow + 32n (chunk sch)
+        // (The instance with far steps has no registers left for address terms hoisted out of the step loop: there the
+        // lane coordinates are taken through `fresh`, which the optimiser cannot see through, so that the few
+        // instructions of an address are redone at each use instead of living in registers that end up in scratch
+        // memory -- a reload inside the loop waits for every outstanding prefetch as well.)
+        auto fresh = [](int x) {
+            if (FARZ) asm volatile("" : "+v"(x));
+            return x;
+        };
         // global -> registers through buffer loads.  The buffer of a step starts at its first row and ends with the
         // last row of the sequence, so rows past the end come back as zeros (hardware range check) with no lane
         // predicated off, and the per-load address arithmetic is scalar.
@@ -561,7 +569,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
             const int el = stage_el + o * RS;  // (o is wave-uniform: one vector add, the row inside the step is an immediate)
 #pragma unroll
             for (int n = 0; n < 2; ++n) {
-                const int at = FARZ ? (o + srow + 32 * n) * RS + sch * 8 : el + 32 * n * RS;
+                const int at = FARZ ? (o + fresh(srow) + 32 * n) * RS + fresh(sch) * 8 : el + 32 * n * RS;
                 if (HAS_C2P) *reinterpret_cast<u32x4*>(&sm.kr[at]) = pre_kr[n];
                 if (HAS_P2C) *reinterpret_cast<u32x4*>(&sm.qr[at]) = pre_qr[n];
             }
@@ -652,17 +660,21 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         };
         auto put_far = [&]() {
             float* const fv = reinterpret_cast<float*>(sm.p);
-            if (hh == 0) {
-                if (HAS_C2P) fv[BN + 32 * w + il] = far_c;
-                if (HAS_P2C && w < 2) fv[32 * w + il] = far_d;
+            const int il_ = fresh(il);
+            if (fresh(hh) == 0) {
+                if (HAS_C2P) fv[BN + 32 * w + il_] = far_c;
+                if (HAS_P2C && w < 2) fv[32 * w + il_] = far_d;
             }
         };
         // Ring slot of the group (rt, a) of batch t: key 64t + ckey - 32rt - 8a with ckey = 60 + 4il - 4hh; `phase` is
         // 64t mod 192.
-        uint16_t* const crow = sm.c + (32 * w + il) * CRS;
-        const int ckey = 60 + 4 * il - 4 * hh;
+        uint16_t* const crow_fixed = sm.c + (32 * w + il) * CRS;
+        const int ckey_fixed = 60 + 4 * il - 4 * hh;
         auto put_c = [&](int phase) {
             if (HAS_C2P) {
+                const int il_ = fresh(il), hh_ = fresh(hh);
+                uint16_t* const crow = FARZ ? sm.c + (32 * w + il_) * CRS : crow_fixed;
+                const int ckey = FARZ ? 60 + 4 * il_ - 4 * hh_ : ckey_fixed;
                 // slot of group (rt, a): y = cb - 32rt - 8a, minus 192 once y reaches 192 -- two base addresses per
                 // step, one compare and one select per store, the distance inside the group as an immediate
                 const int cb = phase + ckey;                    // 56 .. 312
@@ -685,10 +697,11 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         };
         auto put_p = [&]() {
             if (HAS_P2C) {
+                const int il_ = fresh(il), hh_ = fresh(hh);
                 auto put1 = [&](int xt, int jt, const u32x2 (&v)[4]) {
 #pragma unroll
                     for (int a = 0; a < 4; ++a)
-                        *reinterpret_cast<u32x2*>(&sm.p[(32 * jt + il) * PS + 32 * xt + 8 * a + 4 * hh]) = v[a];
+                        *reinterpret_cast<u32x2*>(&sm.p[(32 * jt + il_) * PS + 32 * xt + 8 * a + 4 * hh_]) = v[a];
                 };
                 put1(w + 1, 0, ppk[0]);
                 put1(w + 1, 1, ppk[1]);
