@@ -202,6 +202,7 @@ def test_layer_matches_hf_golden(name, golden_dir):
     (1, 2, 300, 32, 128, None),
     (1, 1, 333, -1, 64, (250,)),
     (1, 1, 1100, 256, 512, None),
+    (1, 1, 2200, 256, 512, (2111,)),        # long enough for the instance with far key steps
 ])
 def test_bf16_fixed_vs_oracle(B, H, L, buckets, max_rel, lengths, force_generic):
     inp = make_inputs(9, B, H, L, 64, buckets, max_rel, dtype=torch.bfloat16, lengths=lengths)
@@ -302,6 +303,7 @@ def test_packed_tile_deal_at_other_grid_sizes():
     (3, 1, 129, 256, 512, (129, 64, 3)),
     (1, 2, 300, 32, 128, None),
     (1, 1, 1100, 256, 512, None),
+    (1, 1, 2200, 256, 512, (2111,)),
 ])
 def test_fp16_fixed_vs_oracle(B, H, L, buckets, max_rel, lengths, force_generic):
     """float16 inputs take the matrix-core kernel too (fp16 MFMA, fp32 accumulation); 11 significant bits give a
