@@ -51,10 +51,11 @@ def prepare(q, k, v, q_pos, k_pos, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max
     B = cu_seqlens_q.numel() - 1
     span = L.att_span(position_buckets, max_relative_distance)
     q, k, v = L.as_rows(q), L.as_rows(k), L.as_rows(v)
-    make = torch.zeros if zero_output else torch.empty
-    o = (torch.zeros_like if zero_output else torch.empty_like)(q)
+    o = torch.empty_like(q)              # q's strides where the kernels can address them, else contiguous
     if not L.rows_ok(o):
-        o = make(q.shape, dtype=q.dtype, device=dev)
+        o = torch.empty(q.shape, dtype=q.dtype, device=dev)
+    if zero_output:
+        o.zero_()
     cu = cu_seqlens_q.to(torch.int32).contiguous()
     if check_cu_seqlens:
         _lib.check_cu_seqlens(cu.cpu().numpy(), T, max(int(max_seqlen_q), 1))
