@@ -552,13 +552,8 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         // a valid row, with no clamping arithmetic.
         const __amdgpu_buffer_rsrc_t lut_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<int*>(p.lut), 0, (lut_max + 1) * 4, RSRC_FLAGS);
         const int srow4 = srow * 4;
-        // (The instance with far steps keeps the plain forms of this lookup, of the ring addressing below and of the
-        // row-maximum exchange: with the cheaper forms its register allocation spills more and the launch is 25 % slower.)
         auto fetch_delta = [&](int s) {
-            if (HAS_POS && FARZ) {
-#pragma unroll
-                for (int n = 0; n < 2; ++n) dl_next[n] = delta_of(row0 - BN * s - (BN - 1) + srow + 32 * n);
-            } else if (HAS_POS) {
+            if (HAS_POS) {
                 const int off = srow4 + (row0 - BN * s - (BN - 1) + p.lut_half) * 4;
                 dl_next[0] = __builtin_amdgcn_raw_buffer_load_b32(lut_rsrc, off, 0, 0);
                 dl_next[1] = __builtin_amdgcn_raw_buffer_load_b32(lut_rsrc, off + 128, 0, 0);
@@ -569,7 +564,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
             const int el = stage_el + o * RS;  // (o is wave-uniform: one vector add, the row inside the step is an immediate)
 #pragma unroll
             for (int n = 0; n < 2; ++n) {
-                const int at = FARZ ? (o + fresh(srow) + 32 * n) * RS + fresh(sch) * 8 : el + 32 * n * RS;
+                const int at = el + 32 * n * RS;
                 if (HAS_C2P) *reinterpret_cast<u32x4*>(&sm.kr[at]) = pre_kr[n];
                 if (HAS_P2C) *reinterpret_cast<u32x4*>(&sm.qr[at]) = pre_qr[n];
             }
@@ -685,13 +680,8 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
 #pragma unroll
                     for (int a = 0; a < 4; ++a) {
                         const int d = 32 * rt + 8 * a;
-                        if (FARZ) {
-                            const int y = cb - d;
-                            *reinterpret_cast<u32x2*>(crow + (y >= CRING ? y - CRING : y)) = cpk[rt][a];
-                        } else {
-                            uint16_t* const base = cb >= CRING + d ? wrapped : flat;
-                            *reinterpret_cast<u32x2*>(base + 56 - d) = cpk[rt][a];
-                        }
+                        uint16_t* const base = cb >= CRING + d ? wrapped : flat;
+                        *reinterpret_cast<u32x2*>(base + 56 - d) = cpk[rt][a];
                     }
             }
         };
@@ -1075,9 +1065,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         for (int jt = 0; jt < 2; ++jt)
 #pragma unroll
             for (int e = 0; e < 16; ++e) mx = fmaxf(mx, s_acc[jt][e]);
-        if (FARZ) {
-            mx = fmaxf(mx, __shfl_xor(mx, 32)) + cadd;
-        } else {
+        {
             float own_or_partner, partner_or_own;
             both_halves(mx, own_or_partner, partner_or_own);
             mx = fmaxf(own_or_partner, partner_or_own) + cadd;
