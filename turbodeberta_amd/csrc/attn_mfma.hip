@@ -1244,7 +1244,7 @@ namespace {
 // Per-device launch facts, looked up once per device under a lock: CU count (rounded down to the 8 XCDs the block
 // ids are dealt over) and, per kernel instance, whether its dynamic-LDS limit has been raised on that device.
 constexpr int kMaxDevices = 64;
-constexpr int FAR_MIN_LEN = 2048;
+constexpr int FAR_MIN_LEN = 1536;
 constexpr int kInstances = 32;
 std::mutex g_dev_mutex;
 int g_cus[kMaxDevices] = {0};
@@ -1285,8 +1285,8 @@ hipError_t tdb_launch_mfma(const TdbKernelParams& whole, int dtype, hipStream_t 
     if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
     const bool c2p = p.pk != nullptr, p2c = p.pq != nullptr;
     // Far key steps only exist in sequences longer than the table's reach; the instance that looks for them carries
-    // both step bodies and its near steps take 1.14x the time, a far step 0.65x.  At length 1024 a quarter of the steps
-    // are far and the plain instance is 9 % faster, at 1536 3 %; from 2048 on (half of the steps) the far instance wins.
+    // both step bodies and its near steps take 1.12x the time, a far step 0.65x.  At length 1024 a quarter of the steps
+    // are far and the plain instance is 7 % faster; at 1536 the far instance wins by 2 %, at 4096 by 13 %.
     const bool farz = (c2p || p2c) && p.L >= FAR_MIN_LEN;
     const int instance = (p.varlen ? 16 : 0) + (farz ? 8 : 0) + (dtype == TDB_F16 ? 4 : 0) + (c2p ? 2 : 0) + (p2c ? 1 : 0);
     const size_t smem = sizeof(Smem);
