@@ -68,10 +68,12 @@ constexpr int CRS = 200;            // its row stride (elements): 400 B, so that
 constexpr int TEAM_MAX = TDB_TEAM;      // workgroups that share one range of a packed launch's tile list
 constexpr int PS = 196;             // row stride (elements) of the p2c scratch [64 keys][191 positions]
 constexpr int RSRC_FLAGS = 0x00020000;   // raw buffer resource, 32-bit data format
-#ifndef TDB_XCD_GROUP
-#define TDB_XCD_GROUP 4
-#endif
-constexpr int XCD_GROUP = TDB_XCD_GROUP;        // query tiles of one (sequence, head) kept on one XCD
+// Query tiles that are neighbours along the query axis (they read the same K and V) are kept on ONE XCD at the same
+// time, in groups of 2^XG tile ids: 4 in the plain instances (the four tiles of a 512-token sequence), 32 -- every CU
+// of an XCD -- in the instances for long sequences, where a (sequence, head) has 12 tiles and more and its keys and
+// values (up to megabytes) then stream through that XCD's L2 once instead of once per group of four
+// (b4 x L4096: 0.512 -> 0.491 ms).
+constexpr int XG_PLAIN = 2, XG_LONG = 5;
 
 struct Smem {
     uint16_t k[2][BN * RS];             // keys of step s live in k[s & 1]
@@ -160,7 +162,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     // the next tile is already on its way from global memory, so that the chain of dependent global reads that
     // starts a tile (sequence length -> delta table -> rows) is only exposed once per workgroup.
     // Virtual block -> (tile, head): consecutive ids go round-robin over the 8 XCDs, each with its own L2; ids are
-    // regrouped so that XCD_GROUP tiles that are neighbours along the query axis -- the tiles that read the same K
+    // regrouped so that G tiles that are neighbours along the query axis -- the tiles that read the same K
     // and V -- run on one XCD and fetch K / V from HBM once instead of once each.
     const int tiles_x = VARLEN ? p.total / BM + p.B : p.B * ((p.L + BM - 1) / BM);
     const int lut_max = 2 * p.lut_half;
@@ -173,7 +175,8 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     };
     auto tile_index = [&](int vb, int& hd, int& tile_id) {   // false: the virtual block has no tile
         const int xcd = vb & 7, slot = vb >> 3;
-        const int v = ((slot / XCD_GROUP) * 8 + xcd) * XCD_GROUP + slot % XCD_GROUP;
+        constexpr int G = 1 << (FARZ ? XG_LONG : XG_PLAIN);
+        const int v = ((slot / G) * 8 + xcd) * G + slot % G;
         if (vb >= nblocks || v >= tiles_x * p.H) return false;
         hd = v / tiles_x;
         tile_id = v - hd * tiles_x;
@@ -1277,8 +1280,6 @@ hipError_t tdb_launch_mfma(const TdbKernelParams& whole, int dtype, hipStream_t 
     }
     const TdbKernelParams& p = whole;
     const int64_t tiles = int64_t(p.varlen ? p.total / BM + p.B : p.B * ((p.L + BM - 1) / BM)) * p.H;
-    const int64_t round = 8 * XCD_GROUP;                 // the id regrouping is a bijection on multiples of this
-    const int nblocks = int((tiles + round - 1) / round * round);
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;
@@ -1288,6 +1289,8 @@ hipError_t tdb_launch_mfma(const TdbKernelParams& whole, int dtype, hipStream_t 
     // both step bodies and its near steps take 1.12x the time, a far step 0.65x.  At length 1024 a quarter of the steps
     // are far and the plain instance is 7 % faster; at 1536 the far instance wins by 2 %, at 4096 by 13 %.
     const bool farz = (c2p || p2c) && p.L >= FAR_MIN_LEN;
+    const int64_t round = int64_t(8) << (farz ? XG_LONG : XG_PLAIN);     // the id regrouping is a bijection on multiples of this
+    const int nblocks = int((tiles + round - 1) / round * round);
     const int instance = (p.varlen ? 16 : 0) + (farz ? 8 : 0) + (dtype == TDB_F16 ? 4 : 0) + (c2p ? 2 : 0) + (p2c ? 1 : 0);
     const size_t smem = sizeof(Smem);
     const void* fn = nullptr;
