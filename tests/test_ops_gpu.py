@@ -263,6 +263,39 @@ def test_bf16_varlen_more_than_64_sequences(force_generic):
             assert torch.equal(part, out[lo:hi]), f"sequences {first}..{first + 49}"
 
 
+def test_repeated_launches_are_bit_identical():
+    """The kernels have no atomics and no order-dependent reduction: the same launch must give the same bits every
+    time.  A difference between repetitions would mean a race between the waves of a workgroup (a missing barrier,
+    an LDS slot overwritten early) that the parity tolerances could hide.  Fixed layout with ragged lengths, packed
+    batch, and a sequence long enough for the instances with far key steps, 100 launches each."""
+    H, D, buckets, max_rel = 12, 64, 256, 512
+    rs = np.random.RandomState(5)
+    lengths = [int(x) for x in rs.randint(16, 513, size=24)]
+    inp = make_inputs(31, len(lengths), H, 512, D, buckets, max_rel, dtype=torch.bfloat16, lengths=lengths)
+    dev = {k: inp[k].to(DEV) for k in ("q", "k", "v", "pk", "pq")}
+    seqlens = torch.tensor(lengths, dtype=torch.int32, device=DEV)
+    packed, cu = pack(inp, lengths)
+    pdev = {k: packed[k].to(DEV) for k in ("q", "k", "v")}
+    cud = cu.to(DEV)
+    long_inp = make_inputs(32, 1, 2, 2304, D, buckets, max_rel, dtype=torch.bfloat16)
+    ldev = {k: long_inp[k].to(DEV) for k in ("q", "k", "v", "pk", "pq")}
+    scale = 1 / math.sqrt(3 * D)
+    runs = {
+        "fixed": lambda: flash_attention_with_disentangled(dev["q"], dev["k"], dev["v"], None, None, False, scale, buckets, max_rel,
+                                                           pos_key_layer=dev["pk"], pos_query_layer=dev["pq"], seqlens_k=seqlens),
+        "packed": lambda: flash_attention_with_disentangled_varlen(pdev["q"], pdev["k"], pdev["v"], None, None, cud, cud, 512, 512,
+                                                                   False, scale, buckets, max_rel, pos_key_layer=dev["pk"],
+                                                                   pos_query_layer=dev["pq"]),
+        "long": lambda: flash_attention_with_disentangled(ldev["q"], ldev["k"], ldev["v"], None, None, False, scale, buckets,
+                                                          max_rel, pos_key_layer=ldev["pk"], pos_query_layer=ldev["pq"]),
+    }
+    for name, run in runs.items():
+        print(f"[case] repeated launches, {name}", flush=True)
+        first = run().clone()
+        for rep in range(100):
+            assert torch.equal(run(), first), f"{name}: launch {rep + 2} differs from the first"
+
+
 def test_packed_tile_deal_at_other_grid_sizes():
     """The packed launch deals its tiles to the persistent workgroups inside the kernel.  Grids of 8, 24 and 40
     workgroups (24 and 40 are not multiples of 16: teams of one) and the full device must all produce every tile:
