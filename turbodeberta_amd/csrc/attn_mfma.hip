@@ -62,10 +62,6 @@ constexpr int WIN = BM + BN;        // ring of staged window rows (one more than
 constexpr int RS = 72;              // LDS row stride (elements) of 64-wide 16-bit rows: 144 B, conflict-free b128
 constexpr int CRING = 192;          // key slots of the c2p ring of one query row
 constexpr int CRS = 200;            // its row stride (elements): 400 B, so that 32 rows read 16 B or write 8 B on distinct banks
-#ifndef TDB_TEAM
-#define TDB_TEAM 2
-#endif
-constexpr int TEAM_MAX = TDB_TEAM;      // workgroups that share one range of a packed launch's tile list
 constexpr int PS = 196;             // row stride (elements) of the p2c scratch [64 keys][191 positions]
 constexpr int RSRC_FLAGS = 0x00020000;   // raw buffer resource, 32-bit data format
 // Query tiles that are neighbours along the query axis (they read the same K and V) are kept on ONE XCD at the same
@@ -83,8 +79,9 @@ struct Smem {
     uint16_t c[BM * CRS];               // c2p ring: row 32w + n belongs to query row0 + 4n + w, slot = key mod 192
     uint16_t p[BN * PS];
     int seq_n[64], seq_lo[64];          // valid length and first token of the first 64 sequences
-    int64_t seq_pre[64];                // packed: inclusive prefix sum of the sequences' tile costs (one head)
-    int64_t deal[NTHREADS / 64][TEAM_MAX + 5];     // packed: state of the tile deal, one copy per wave
+    int srt_seq[64];                    // packed: the sequences in order of decreasing length (ties: lower index first)
+    int64_t seq_pre[64];                // packed: inclusive prefix sum, in that order, of the sequences' tile counts (all heads)
+    int deal_round[NTHREADS / 64];      // packed: how many tiles this workgroup has taken so far, one copy per wave
 };
 
 // The two 16-bit element types the kernel is instantiated for: what differs is the MFMA and the float conversion.
@@ -171,7 +168,6 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     struct Tile {
         int vb, head, b, row0, len;       // vb < 0: no tile
         int64_t tok0;
-        int64_t cost;                     // balanced walk: cost coordinate of the tile (see below)
     };
     auto tile_index = [&](int vb, int& hd, int& tile_id) {   // false: the virtual block has no tile
         const int xcd = vb & 7, slot = vb >> 3;
@@ -193,24 +189,20 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         return int64_t((uint64_t(uint32_t(hi)) << 32) | uint32_t(lo));
     };
     auto tiles_of = [](int n) { return (n + BM - 1) / BM; };
-    auto cost_of = [](int n) { return int64_t(8 * ((n + BN - 1) / BN) + 24); };
-    // Packed launches (at most 64 sequences: the launcher splits larger batches) use a cost-balanced walk instead of
-    // the strided one of the fixed layout: tiles differ in length by up to 8x, so a TEAM of workgroups takes a
-    // CONTIGUOUS range of the tile list (heads outermost, then sequences, then the query tiles of a sequence) whose
-    // summed cost is its share of the total.  The cost of a tile is 8 * (its key steps) + 24, in eighths of a key
-    // step (24: what a tile costs beside its steps; measured, the launch time is flat between 24 and 32 and 2.5 %
-    // higher at 13 or 40).  Every wave derives the
-    // same ranges from the sequence boundaries; a tile belongs to the team whose cost interval holds the tile's
-    // start coordinate.  A team is TEAM workgroups that sit on one XCD (block ids go round-robin over the 8 XCDs);
-    // inside a team the tiles are dealt in list order, each to the member with the least cost so far -- what a
-    // shared work queue would do, computed by every member for itself.  The query tiles of one (sequence, head),
-    // neighbours in the list, therefore run at the same time on CUs that share an L2 and read K and V from HBM
-    // once, not once per tile.  (Measured on 64 sequences of 16..512 tokens: L2 fetches are 2.9x the algorithmic
-    // bytes with one range per workgroup dealt round-robin over the XCDs, 2.0x with each XCD's ranges adjacent, 1.2x
-    // for teams of 2, 1.1x for teams of 4 -- but the launch takes 2 % / 12 % longer with teams of 2 / 4 than with
-    // none, so teams are pairs.)  Cost coordinates are 64-bit: one sequence of 2^20 tokens alone costs 2^30.  The
-    // state of the deal (next tile of the list, cost per member) lives in LDS, one copy per wave: it is touched once
-    // per tile and would otherwise occupy registers all through the key steps.
+    // Packed launches (at most 64 sequences: the launcher splits larger batches) deal their tiles by cost instead of
+    // the strided walk of the fixed layout: a tile costs about 3 key steps plus one per 64 keys of its sequence, so
+    // tiles differ by up to 3x.  The tiles are listed by decreasing length of their sequence (then head, then query
+    // tile) and dealt to the G workgroups back and forth: round j hands tiles j*G .. j*G+G-1 out in ascending order
+    // of the workgroup number when j is even, in descending order when it is odd, so that whoever got the costlier
+    // tile of one round gets the cheaper one of the next, and the last, incomplete round -- the cheapest tiles --
+    // goes to the workgroups that have the least so far.  Every workgroup derives its own tiles from the sequence
+    // boundaries alone (a rank per sequence, a prefix sum of tile counts in rank order, one search per tile); nothing
+    // is shared between workgroups.  (64 sequences of 16..512 tokens: the most loaded workgroup carries 1.04-1.07x
+    // the mean; contiguous cost-balanced ranges of the unsorted list, the earlier scheme, 1.11x and a 10 % longer
+    // launch.)  Workgroups are numbered for the deal so that neighbours sit on ONE XCD (block ids go round-robin
+    // over the 8 XCDs): the query tiles of one (sequence, head), neighbours in the list, then run at the same time
+    // on CUs that share an L2 and read K and V from HBM once, not once per tile.  The round counter lives in LDS,
+    // one copy per wave: it is touched once per tile and would otherwise occupy a register all through the key steps.
     constexpr bool balanced = VARLEN;
     {
         int n = p.L, lo = 0;
@@ -225,14 +217,26 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         }
         sm.seq_n[l] = n;
         if (VARLEN) {                     // (the fixed layout's walk needs the lengths only)
-            int64_t pre = tiles_of(n) * cost_of(n);                      // inclusive prefix sum over the wave
+            sm.seq_lo[l] = lo;
+            // Rank of this lane's sequence by decreasing length (ties: lower index first); the sequence and the tile
+            // count (all heads) that belong at rank l travel to lane l inside the wave, and the tile counts become an
+            // inclusive prefix sum in that order.  (All eight waves write the same final values into the shared
+            // arrays and each reads back what it wrote itself; nothing intermediate goes through them -- a second
+            // wave could be anywhere in this sequence.)
+            int rank = 0;
+            for (int b2 = 0; b2 < 64; ++b2) {
+                const int n2 = sm.seq_n[b2];
+                rank += (n2 > n || (n2 == n && b2 < l)) ? 1 : 0;
+            }
+            const int seq_here = __builtin_amdgcn_ds_permute(rank * 4, l);
+            int64_t cnt = int64_t(__builtin_amdgcn_ds_permute(rank * 4, tiles_of(n))) * p.H;
 #pragma unroll
             for (int d = 1; d < 64; d <<= 1) {
-                const int64_t up = __shfl_up(pre, d);
-                if (l >= d) pre += up;
+                const int64_t up = __shfl_up(cnt, d);
+                if (l >= d) cnt += up;
             }
-            sm.seq_lo[l] = lo;
-            sm.seq_pre[l] = pre;
+            sm.srt_seq[l] = seq_here;
+            sm.seq_pre[l] = cnt;
         }
     }
     // fixed layout: tile_id -> (sequence, first row, valid length); same map as tdb_locate_tile
@@ -244,124 +248,40 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         t0 = 0;
         return true;
     };
-    constexpr int TEAM = TEAM_MAX;
-    // deal state of this wave: cost per member, then [+0] cost coordinate of the next tile of the list, [+1] end of
-    // the team's cost interval, [+2] head << 32 | sequence, [+3] tile within the sequence (-1: the list is
-    // exhausted), [+4] length << 32 | first token of that sequence
-    int64_t* const deal = sm.deal[wave];
-    // Moves (head, sequence, tile) forward until it names an existing tile of the team's interval; t.cost is its
-    // start coordinate.  t.len > 0: length and first token of sequence t.b are already in t (the common case, the
-    // next tile of the same sequence, then reads nothing).
-    auto settle = [&](Tile t, int tile_in_seq, int64_t cost_end) {
-        while (t.head < p.H) {
-            const int n = t.len > 0 ? t.len : lds_int(&sm.seq_n[t.b]);
-            if (tile_in_seq < tiles_of(n)) {
-                if (t.len <= 0) t.tok0 = lds_int(&sm.seq_lo[t.b]);
-                t.row0 = tile_in_seq * BM;
-                t.len = n;
-                t.vb = t.cost < cost_end ? 0 : -1;
-                return t;
-            }
-            const int64_t cost_per_head = lds_i64(&sm.seq_pre[63]);
-            const unsigned long long have = __builtin_amdgcn_ballot_w64(sm.seq_n[l] > 0);
-            const unsigned long long later = t.b >= 63 ? 0ull : have & ~((2ull << t.b) - 1ull);
-            tile_in_seq = 0;
-            t.len = 0;
-            if (later) {
-                t.b = __builtin_ctzll(later);
-            } else {                      // next head (a launch without any tile never gets here: cost_per_head > 0)
-                t.head += 1;
-                t.b = __builtin_ctzll(have);
-                t.cost = t.head * cost_per_head;
-            }
-        }
-        t.vb = -1;
-        return t;
-    };
     auto no_tile = []() {
         Tile t;
         t.vb = -1;
         t.head = t.b = t.row0 = t.len = 0;
-        t.cost = 0;
         t.tok0 = 0;
         return t;
     };
-    auto take = [&]() {                   // deals tiles of the team's list until one falls to this workgroup
-        const int team_size = gridDim.x % (8 * TEAM) == 0 ? TEAM : 1;
-        const int member = int(blockIdx.x >> 3) % team_size;
-        int64_t load[TEAM];
-#pragma unroll
-        for (int m = 0; m < TEAM; ++m) load[m] = lds_i64(&deal[m]);
-        const int64_t cost_end = lds_i64(&deal[TEAM_MAX + 1]);
-        const int64_t where = lds_i64(&deal[TEAM_MAX + 2]);
-        const int tile_in_seq = int(lds_i64(&deal[TEAM_MAX + 3]));
-        const int64_t seq = lds_i64(&deal[TEAM_MAX + 4]);
-        Tile cursor = no_tile(), mine = no_tile();
-        cursor.cost = lds_i64(&deal[TEAM_MAX + 0]);
-        if (tile_in_seq >= 0) {
-            cursor.head = int(where >> 32);
-            cursor.b = int(where & 0xffffffff);
-            cursor.len = int(seq >> 32);
-            cursor.tok0 = int(seq & 0xffffffff);
-            cursor.row0 = tile_in_seq * BM;
-            cursor.vb = 0;
-        }
-        while (cursor.vb >= 0) {
-            const Tile t = cursor;
-            int m = 0;
-            int64_t least = load[0];
-#pragma unroll
-            for (int i = 1; i < TEAM; ++i)
-                if (load[i] < least) {
-                    least = load[i];
-                    m = i;
-                }
-            const int64_t c = cost_of(t.len);
-#pragma unroll
-            for (int i = 0; i < TEAM; ++i) load[i] += i == m ? c : 0;
-            cursor.cost += c;
-            cursor = settle(cursor, t.row0 / BM + 1, cost_end);
-            if (m == member) {
-                mine = t;
-                break;
-            }
-        }
-#pragma unroll
-        for (int m = 0; m < TEAM; ++m) deal[m] = load[m];
-        deal[TEAM_MAX + 0] = cursor.cost;
-        deal[TEAM_MAX + 2] = (int64_t(cursor.head) << 32) | int64_t(uint32_t(cursor.b));
-        deal[TEAM_MAX + 3] = cursor.vb >= 0 ? cursor.row0 / BM : -1;
-        deal[TEAM_MAX + 4] = (int64_t(cursor.len) << 32) | int64_t(uint32_t(cursor.tok0));
-        return mine;
+    // Tile j of this workgroup in the back-and-forth deal (gridDim.x is a multiple of 8).
+    auto dealt_tile = [&](int j) {
+        const int64_t G = gridDim.x, g = int64_t(blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+        const int64_t k = int64_t(j) * G + ((j & 1) ? G - 1 - g : g);
+        Tile t = no_tile();
+        if (k >= lds_i64(&sm.seq_pre[63])) return t;
+        const unsigned long long owners = __builtin_amdgcn_ballot_w64(sm.seq_pre[l] > k);
+        const int r = __builtin_amdgcn_readfirstlane(__builtin_ctzll(owners));
+        t.b = lds_int(&sm.srt_seq[r]);
+        t.len = lds_int(&sm.seq_n[t.b]);
+        t.tok0 = lds_int(&sm.seq_lo[t.b]);
+        const int per_head = tiles_of(t.len);
+        if (owners == 0 || per_head <= 0) return no_tile();
+        const int within = int(k - (lds_i64(&sm.seq_pre[r]) - int64_t(per_head) * p.H));
+        t.head = within / per_head;
+        t.row0 = (within - t.head * per_head) * BM;
+        t.vb = (within >= 0 && t.head < p.H) ? 0 : -1;     // (always true for a consistent prefix: no tile rather than a stray address)
+        return t;
+    };
+    auto take = [&]() {
+        const int j = lds_int(&sm.deal_round[wave]) + 1;
+        sm.deal_round[wave] = j;
+        return dealt_tile(j);
     };
     auto first_balanced = [&]() {
-        const int team_size = gridDim.x % (8 * TEAM) == 0 ? TEAM : 1;
-#pragma unroll
-        for (int m = 0; m < TEAM; ++m) deal[m] = m < team_size ? 0 : INT64_MAX;   // members that do not exist: never the least
-        deal[TEAM_MAX + 3] = -1;
-        const int64_t cost_per_head = lds_i64(&sm.seq_pre[63]);
-        if (cost_per_head <= 0) return no_tile();
-        const int64_t teams = gridDim.x / team_size;
-        const int64_t team = int64_t(blockIdx.x & 7) * (teams / 8) + int64_t(blockIdx.x >> 3) / team_size;   // gridDim.x is a multiple of 8
-        const int64_t total = cost_per_head * p.H;           // < 2^30 * 64 * 2^16: no overflow; the products below
-        const int64_t start = total / teams * team + total % teams * team / teams;   // stay below 2^63 too
-        const int64_t cost_end = total / teams * (team + 1) + total % teams * (team + 1) / teams;
-        Tile t = no_tile();
-        t.head = int(start / cost_per_head);
-        const int64_t rem = start - t.head * cost_per_head;
-        const unsigned long long owners = __builtin_amdgcn_ballot_w64(sm.seq_pre[l] > rem);
-        t.b = __builtin_amdgcn_readfirstlane(__builtin_ctzll(owners));
-        const int n = lds_int(&sm.seq_n[t.b]);
-        const int64_t before = lds_i64(&sm.seq_pre[t.b]) - tiles_of(n) * cost_of(n);
-        const int tile_in_seq = int((rem - before + cost_of(n) - 1) / cost_of(n));     // first tile starting at or after rem
-        t.cost = t.head * cost_per_head + before + tile_in_seq * cost_of(n);
-        t = settle(t, tile_in_seq, cost_end);
-        deal[TEAM_MAX + 0] = t.cost;
-        deal[TEAM_MAX + 1] = cost_end;
-        deal[TEAM_MAX + 2] = (int64_t(t.head) << 32) | int64_t(uint32_t(t.b));
-        deal[TEAM_MAX + 3] = t.vb >= 0 ? t.row0 / BM : -1;
-        deal[TEAM_MAX + 4] = (int64_t(t.len) << 32) | int64_t(uint32_t(t.tok0));
-        return take();
+        sm.deal_round[wave] = 0;
+        return dealt_tile(0);
     };
     // First tile with live query rows among the virtual blocks vb, vb + gridDim.x, ...; vb = -1 if there is none.
     // Tiles that hold only padded query rows (fixed layout) get their zeros here, from whoever looks them up:
@@ -370,7 +290,6 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         Tile t;
         t.vb = -1;
         t.head = t.b = t.row0 = t.len = 0;
-        t.cost = 0;
         t.tok0 = 0;
         for (; vb < nblocks; vb += gridDim.x) {
             int hd, tile_id;
@@ -928,7 +847,6 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     Tile nxt;                             // the tile after the current one (looked up while a tile opens)
     nxt.vb = -1;
     nxt.head = nxt.b = nxt.row0 = nxt.len = 0;
-    nxt.cost = 0;
     nxt.tok0 = 0;
     int cphase = 0;                       // ring slot of the first key of the step: 64s mod 192
     bool far_cur = false;                 // whether the step about to run is far; far_open: step 0 of the tile to open
