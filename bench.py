@@ -7,8 +7,12 @@ A "step" is one attention forward over one batch of synthetic DeBERTa-v3-base at
   fixed   batch 32 x seq 512, right-padded, valid lengths uniform in [384, 512]   (headline `value`)
   varlen  64 sequences with lengths uniform in [16, 512], packed with cu_seqlens  (reported beside it)
   long    batch 4 x seq 4096, full mask, and its packed variant (8 sequences U[1024, 4096])   (`long`, `long_varlen`)
-  generic the vector-ALU kernel that serves float32 inputs and the strip-taking signature: the attention of the
-          config-1 layer (batch 2 x seq 128, float32) and a strip-mode call at batch 8 x seq 256 in bf16   (`generic`)
+  strips  the reference's own call signature -- c2p / p2c strips [B, H, L, 2*span] computed by the caller -- on the
+          matrix-core kernel: batch 8 x seq 256 and batch 32 x seq 512, bf16, priced against HBM (the strips are
+          most of the bytes)   (`strips`)
+  generic the vector-ALU kernel that serves float32 inputs and what the matrix-core kernel does not take: the
+          attention of the config-1 layer (batch 2 x seq 128, float32), and the batch 8 x seq 256 strip call forced
+          onto it for comparison   (`generic`)
 
 Prints ONE JSON line.  `value` is algorithmic attention TFLOP/s of the fixed workload over the timed
 region; FLOPs per sequence of valid length l and per head:  4*l*l*d (QK^T + PV) + 4*l*W*d (c2p + p2c),
@@ -155,28 +159,58 @@ def build_long(dev, B=4, L=4096):
     return plan, np.full(B, L)
 
 
+def _strip_call(dev, w, g, B, L, dt, force_generic=False):
+    """The reference's literal call shape: c2p / p2c strips [B, H, L, 2*span] computed by the caller (model.py:122-137
+    of the reference), full mask."""
+    from turbodeberta_amd.ops import flash_attention as fa
+    lin = torch.nn.functional.linear
+    hidden = torch.randn(B, L, HID, generator=g, device=dev, dtype=torch.float32).to(dt)
+    heads = lambda x: x.view(B, L, H, D).permute(0, 2, 1, 3)
+    q, k, v = (heads(lin(hidden, w[n].to(dt))) for n in ("wq", "wk", "wv"))
+    pk, pq = (t.to(dt) for t in position_tables(w))
+    c2p = torch.matmul(q, pk.transpose(-1, -2)[None])
+    p2c = torch.matmul(k, pq.transpose(-1, -2)[None])
+    return fa.prepare(q, k, v, c2p, p2c, False, 1.0 / math.sqrt(3 * D), BUCKETS, MAX_REL, force_generic=force_generic)
+
+
 def build_generic(dev):
-    """The two callers of the vector-ALU kernel: (a) the attention of the config-1 layer -- batch 2 x seq 128, 12 heads,
-    float32, full mask; (b) the reference's literal call shape -- c2p / p2c strips [B, H, L, 2*span] computed by the
-    caller (model.py:122-137 of the reference) -- at batch 8 x seq 256 in bf16."""
+    """The vector-ALU kernel: (a) the attention of the config-1 layer -- batch 2 x seq 128, 12 heads, float32, full
+    mask, the case it exists for; (b) the strip call at batch 8 x seq 256 in bf16 forced onto it (without the flag that
+    call runs on the matrix cores: `build_strips`)."""
     from turbodeberta_amd.ops import flash_attention as fa
     w, g = make_weights(dev)
     lin = torch.nn.functional.linear
-    out = {}
-    for name, (B, L, dt) in {"config1_fp32": (2, 128, torch.float32), "strips_bf16": (8, 256, torch.bfloat16)}.items():
-        hidden = torch.randn(B, L, HID, generator=g, device=dev, dtype=torch.float32).to(dt)
-        heads = lambda x: x.view(B, L, H, D).permute(0, 2, 1, 3)
-        q, k, v = (heads(lin(hidden, w[n].to(dt))) for n in ("wq", "wk", "wv"))
-        pk, pq = (t.to(dt) for t in position_tables(w))
-        if name == "strips_bf16":
-            c2p = torch.matmul(q, pk.transpose(-1, -2)[None])
-            p2c = torch.matmul(k, pq.transpose(-1, -2)[None])
-            plan = fa.prepare(q, k, v, c2p, p2c, False, 1.0 / math.sqrt(3 * D), BUCKETS, MAX_REL)
-        else:
-            plan = fa.prepare(q, k, v, None, None, False, 1.0 / math.sqrt(3 * D), BUCKETS, MAX_REL,
-                              pos_key_layer=pk, pos_query_layer=pq)
-        out[name] = (plan, np.full(B, L))
-    return out
+    B, L, dt = 2, 128, torch.float32
+    hidden = torch.randn(B, L, HID, generator=g, device=dev, dtype=torch.float32).to(dt)
+    heads = lambda x: x.view(B, L, H, D).permute(0, 2, 1, 3)
+    q, k, v = (heads(lin(hidden, w[n].to(dt))) for n in ("wq", "wk", "wv"))
+    pk, pq = (t.to(dt) for t in position_tables(w))
+    plan = fa.prepare(q, k, v, None, None, False, 1.0 / math.sqrt(3 * D), BUCKETS, MAX_REL,
+                      pos_key_layer=pk, pos_query_layer=pq)
+    return {"config1_fp32": (plan, np.full(B, L)),
+            "strips_bf16_forced": (_strip_call(dev, w, g, 8, 256, torch.bfloat16, force_generic=True), np.full(8, 256))}
+
+
+def build_strips(dev):
+    """The strip call on the matrix-core kernel at batch 8 x seq 256 and at the headline shape, batch 32 x seq 512."""
+    w, g = make_weights(dev)
+    return {"b8xL256": (_strip_call(dev, w, g, 8, 256, torch.bfloat16), np.full(8, 256)),
+            "b32xL512": (_strip_call(dev, w, g, 32, 512, torch.bfloat16), np.full(32, 512))}
+
+
+def strip_bytes(lengths) -> float:
+    """Algorithmic bytes of a strip call: q, k, v read and o written once, plus every strip element that some score
+    position addresses -- row i of either strip is read at the columns delta(i - j), j < l, a contiguous range because
+    delta is monotone."""
+    from turbodeberta_amd import _lib
+    tot = 0.0
+    for l in lengths:
+        l = int(l)
+        lut = _lib.delta_table(l, BUCKETS, MAX_REL).astype(np.int64)       # entry r + l - 1
+        i = np.arange(l)
+        cols = lut[i + l - 1] - lut[i] + 1                                   # delta(i - 0) - delta(i - (l - 1)) + 1
+        tot += 2.0 * 4 * l * H * D + 2 * 2.0 * H * float(cols.sum())
+    return tot
 
 
 def build_varlen(dev, n_seq=64, lo=16, hi=512):
@@ -353,8 +387,8 @@ def main():
                     help="untimed launches of the workload for this many ms before the warm-up, to get past the clock "
                          "ramp that follows an idle period (0 switches it off)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--workload", choices=["all", "both", "fixed", "varlen", "long", "generic"], default="all",
-                    help="all = fixed + varlen + long + long_varlen + generic; both = fixed + varlen")
+    ap.add_argument("--workload", choices=["all", "both", "fixed", "varlen", "long", "strips", "generic"], default="all",
+                    help="all = fixed + varlen + long + long_varlen + strips + generic; both = fixed + varlen")
     ap.add_argument("--with-model", action="store_true",
                     help="add the end-to-end forward of a v3-large-shaped model (fused attention vs Hugging Face eager "
                          "attention on the same GPU) to the JSON line as \"model\"")
@@ -383,23 +417,27 @@ def main():
            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic"}
     spent_prewarm = []
 
-    def measure(plan, lengths, name, kernel, peak=PEAK_BF16_TFLOPS, bound="mfma", steps=None):
+    def measure(plan, lengths, name, kernel, peak=PEAK_BF16_TFLOPS, bound="mfma", steps=None, nbytes=None):
         steps = steps or args.steps
         wall_ms, mean_ms, med_ms, min_ms, spent = time_steps(plan, steps, args.warmup, args.prewarm_ms)
         spent_prewarm.append(spent)
         fl = flops_of(lengths)
-        ach = fl / (mean_ms * 1e-3) / 1e12
+        nbytes = algorithmic_bytes(lengths) if nbytes is None else nbytes
+        if bound == "hbm":                                         # priced by bytes: GB/s against the HBM peak
+            ach, peak, unit = nbytes / (mean_ms * 1e-3) / 1e9, PEAK_HBM_GBS, "GB/s"
+        else:
+            ach, unit = fl / (mean_ms * 1e-3) / 1e12, "TFLOP/s"
         traffic, traffic_source, traffic_stale = recorded_traffic(name)
         return {
             "value": round(fl / (wall_ms * 1e-3) / 1e12, 2), "ms_per_step": round(wall_ms, 4), "steps": steps,
             "tokens_per_s": round(float(lengths.sum()) / (wall_ms * 1e-3), 1),
             "core_tflops": round(H * sum(4.0 * int(l) ** 2 * D for l in lengths) / (wall_ms * 1e-3) / 1e12, 2),
-            "roofline": {"bound": bound, "achieved": round(ach, 2), "peak": peak, "unit": "TFLOP/s",
+            "roofline": {"bound": bound, "achieved": round(ach, 2), "peak": peak, "unit": unit,
                          "frac": round(ach / peak, 4), "traffic": traffic, "traffic_source": traffic_source, "traffic_stale": traffic_stale,
                          "kernel": kernel,
                          "kernel_ms_mean": round(mean_ms, 4), "kernel_ms_pair_median": round(med_ms, 4),
-                         "kernel_ms_pair_min": round(min_ms, 4), "algorithmic_gflop": round(fl / 1e9, 3), "algorithmic_bytes": algorithmic_bytes(lengths),
-                         "hbm_gbs_algorithmic": round(algorithmic_bytes(lengths) / (mean_ms * 1e-3) / 1e9, 1)},
+                         "kernel_ms_pair_min": round(min_ms, 4), "algorithmic_gflop": round(fl / 1e9, 3), "algorithmic_bytes": nbytes,
+                         "hbm_gbs_algorithmic": round(nbytes / (mean_ms * 1e-3) / 1e9, 1)},
         }
 
     res_fixed = res_var = None
@@ -421,13 +459,23 @@ def main():
         extra["long_varlen"] = {"workload": "8 packed sequences, lengths U[1024,4096] seed 0, total tokens %d" % int(lengths_lv.sum()),
                                 **measure(plan_lv, lengths_lv, "long_varlen", "attn_mfma_kernel<c2p,p2c>", steps=few)}
         del plan_lv
+    if args.workload in ("all", "strips"):
+        extra["strips"] = {}
+        for name, (pl, ln) in build_strips(dev).items():
+            extra["strips"][name] = {"workload": "strip-taking signature (c2p / p2c strips [B,H,L,512] from the caller), "
+                                                 "batch %d x seq %d, full mask, bf16" % (len(ln), int(ln[0])),
+                                     **measure(pl, ln, "strips_" + name, "attn_mfma_kernel<c2p,p2c,strips>", bound="hbm",
+                                               nbytes=strip_bytes(ln))}
+            del pl
+        torch.cuda.empty_cache()
     if args.workload in ("all", "generic"):
         notes = {"config1_fp32": "attention of the config-1 layer: batch 2 x seq 128, 12 heads x 64, float32, fused tables",
-                 "strips_bf16": "strip-taking signature (c2p / p2c strips [B,H,L,512] from the caller), batch 8 x seq 256, bf16"}
+                 "strips_bf16_forced": "strip-taking signature, batch 8 x seq 256, bf16, forced onto the vector-ALU kernel "
+                                       "(without the flag it runs on the matrix cores: `strips.b8xL256`)"}
         extra["generic"] = {name: {"workload": notes[name],
                                    **measure(pl, ln, name, "attn_generic_kernel", peak=PEAK_FP32_VALU_TFLOPS, bound="valu")}
                             for name, (pl, ln) in build_generic(dev).items()}
-    head = res_fixed or res_var or extra.get("long") or next(iter(extra["generic"].values()))
+    head = res_fixed or res_var or extra.get("long") or next(iter((extra.get("strips") or extra["generic"]).values()))
     out.update({"value": head["value"], "ms_per_step": head["ms_per_step"], "tokens_per_s": head["tokens_per_s"],
                 "core_tflops": head["core_tflops"], "roofline": head["roofline"]})
     out["config"] = {"workload": ("fixed b32xL512, valid lengths U[384,512] seed 0" if res_fixed else

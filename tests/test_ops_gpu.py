@@ -367,6 +367,104 @@ def test_fp16_varlen_matrix_core_equals_vector_alu():
         assert_close_bf16(outs[-1], ref, f"fp16 varlen generic={gen}", tol=2e-3)
 
 
+# ------------------------------------------------------------------ 16-bit strips (the reference's own operator signature)
+
+def _strips(inp, types=("c2p", "p2c")):
+    """The strips the reference glue hands to its kernel (model.py:122-125, :146-148): Q.K_r^T and K.Q_r^T, computed
+    and rounded in the element type."""
+    c2p = torch.matmul(inp["q"], inp["pk"].transpose(-1, -2)[None]) if "c2p" in types else None
+    p2c = torch.matmul(inp["k"], inp["pq"].transpose(-1, -2)[None]) if "p2c" in types else None
+    return c2p, p2c
+
+
+def _run_strips(inp, c2p, p2c, buckets, max_rel, n_terms=2, **kw):
+    dev = lambda t: None if t is None else t.to(DEV)
+    D = inp["q"].shape[-1]
+    print(f"[case] fixed strips q={tuple(inp['q'].shape)} {inp['q'].dtype} buckets={buckets} max_rel={max_rel} "
+          f"c2p={c2p is not None} p2c={p2c is not None} kw={kw}", flush=True)
+    out = flash_attention_with_disentangled(dev(inp["q"]), dev(inp["k"]), dev(inp["v"]), dev(c2p), dev(p2c), False,
+                                            1.0 / math.sqrt(D * (1 + n_terms)), buckets, max_rel,
+                                            seqlens_k=dev(inp.get("lengths")), **kw)
+    torch.cuda.synchronize()
+    return out.cpu()
+
+
+@pytest.mark.parametrize("force_generic", [False, True])
+@pytest.mark.parametrize("B,H,L,buckets,max_rel,lengths", [
+    (2, 12, 128, 256, 512, None),
+    (2, 2, 512, 256, 512, (512, 389)),
+    (1, 2, 1, 256, 512, None),
+    (3, 1, 129, 256, 512, (129, 64, 3)),
+    (1, 2, 300, 32, 128, None),
+    (1, 1, 333, -1, 64, (250,)),
+    (1, 1, 1100, 256, 512, None),
+])
+def test_bf16_strips_fixed_vs_oracle(B, H, L, buckets, max_rel, lengths, force_generic):
+    """Strips in bf16, as Hugging Face's eager code holds them before its gather: the bf16 eager oracle is the same
+    computation, the fp32 oracle differs by the rounding of the strips."""
+    inp = make_inputs(21, B, H, L, 64, buckets, max_rel, dtype=torch.bfloat16, lengths=lengths)
+    c2p, p2c = _strips(inp)
+    out = _run_strips(inp, c2p, p2c, buckets, max_rel, force_generic=force_generic)
+    ref32 = oracle_fixed(inp, buckets, max_rel, dtype=torch.float32)
+    assert_close_bf16(out, ref32, "bf16 strips vs fp32 oracle on rounded inputs", tol=1e-2)
+    if L <= 512:
+        ref16 = oracle_fixed(inp, buckets, max_rel, dtype=torch.bfloat16)
+        assert_close_bf16(out, ref16, "bf16 strips vs bf16 eager oracle")
+    if lengths is not None:
+        for b, n in enumerate(lengths):
+            assert torch.all(out[b, :, n:] == 0)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("types", [("c2p", "p2c"), ("c2p",), ("p2c",)])
+def test_random_strips_matrix_core_equals_vector_alu(types, dtype):
+    """Strips of independent random values (no table behind them): every (row, column) of a strip holds its own
+    number, so a wrong row, a wrong column or a value filed under the wrong key moves the output.  The vector-ALU
+    kernel, pinned against the oracle in fp32, reads the same strips element by element."""
+    B, H, L, buckets, max_rel = 2, 3, 400, 256, 512
+    inp = make_inputs(22, B, H, L, 64, buckets, max_rel, dtype=dtype, lengths=(400, 213))
+    g = torch.Generator().manual_seed(23)
+    c2p = (torch.randn(B, H, L, 2 * buckets, generator=g) * 4).to(dtype) if "c2p" in types else None
+    p2c = (torch.randn(B, H, L, 2 * buckets, generator=g) * 4).to(dtype) if "p2c" in types else None
+    fast = _run_strips(inp, c2p, p2c, buckets, max_rel, n_terms=len(types))
+    slow = _run_strips(inp, c2p, p2c, buckets, max_rel, n_terms=len(types), force_generic=True)
+    assert_close_bf16(fast, slow, f"random strips {types} {dtype}", tol=4e-3 if dtype == torch.float16 else 1e-2)
+    # and against the definition, on the valid rows of the first sequence
+    f = lambda t: t[0].float()
+    idx = O.relative_position_index(400, 400, buckets, max_rel)                   # [L, L] columns delta(i - j)
+    s = torch.einsum("hid,hjd->hij", f(inp["q"]), f(inp["k"]))
+    if c2p is not None:
+        s = s + torch.gather(f(c2p), 2, idx[None].expand(H, -1, -1))
+    if p2c is not None:
+        s = s + torch.gather(f(p2c), 2, idx.t()[None].expand(H, -1, -1)).transpose(1, 2)
+    ref = torch.softmax(s / math.sqrt(64 * (1 + len(types))), -1) @ f(inp["v"])
+    assert_close_bf16(fast[0], ref, f"random strips {types} {dtype} vs definition", tol=1e-2)
+
+
+def test_bf16_strips_varlen_vs_oracle():
+    H, D, buckets, max_rel = 4, 64, 256, 512
+    rs = np.random.RandomState(1)
+    lengths = [int(x) for x in rs.randint(16, 513, size=10)] + [1, 128, 129, 0, 64]
+    inp = make_inputs(24, len(lengths), H, max(lengths), D, buckets, max_rel, dtype=torch.bfloat16)
+    packed, cu = pack(inp, lengths)
+    f = lambda t: t.float()
+    ref = O.attention_varlen(f(packed["q"]), f(packed["k"]), f(packed["v"]), f(inp["pk"]), f(inp["pq"]), cu,
+                             position_buckets=buckets, max_relative_positions=max_rel)
+    c2p = torch.einsum("thd,hmd->thm", packed["q"], inp["pk"])
+    p2c = torch.einsum("thd,hmd->thm", packed["k"], inp["pq"])
+    outs = []
+    for force_generic in (False, True):
+        print(f"[case] bf16 varlen strips generic={force_generic} lengths={lengths}", flush=True)
+        out = flash_attention_with_disentangled_varlen(
+            packed["q"].to(DEV), packed["k"].to(DEV), packed["v"].to(DEV), c2p.to(DEV), p2c.to(DEV), cu.to(DEV),
+            cu.to(DEV), max(lengths), max(lengths), False, 1 / math.sqrt(3 * D), buckets, max_rel,
+            force_generic=force_generic)
+        torch.cuda.synchronize()
+        assert_close_bf16(out.cpu(), ref, f"bf16 varlen strips generic={force_generic}", tol=1e-2)
+        outs.append(out.cpu())
+    assert_close_bf16(outs[0], outs[1], "bf16 varlen strips, matrix cores vs vector ALUs", tol=4e-3)
+
+
 def test_backward_raises_like_the_reference():
     q = torch.randn(1, 1, 8, 64, device=DEV, requires_grad=True)
     out = flash_attention_with_disentangled(q, q, q, None, None)

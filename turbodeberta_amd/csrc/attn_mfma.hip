@@ -33,6 +33,12 @@
 //         P'[j][i - j - B_s], which becomes the initial value of the S^T accumulator.
 // Together: S[i,j] = Q_i.K_j + Q_i.K_r[delta(i-j)] + K_j.Q_r[delta(i-j)], the Hugging Face eager
 // definition (modeling_deberta_v2.py:317-324, :337-343).
+//
+// Callers of the reference's own signature hold the position products already, as strips
+// c2p[i][x] = Q_i.K_r[x] and p2c[j][x] = K_j.Q_r[x] over all 2*span table rows x.  The strip instances
+// keep the score waves as they are and give the position waves a different job: no tables, no
+// products -- they gather c2p[i][delta(i-j)] and p2c[j][delta(i-j)] from global memory into the same
+// ring and scratch layouts, one key step ahead, between the same barriers.
 #include <atomic>
 #include <mutex>
 #include <type_traits>
@@ -133,12 +139,13 @@ __device__ __forceinline__ void phase_barrier() {
     __builtin_amdgcn_sched_barrier(0);
 }
 
-// Template parameters: which position terms exist, the element type, whether far key steps are looked for, and the
-// layout (VARLEN: packed sequences).  The layout is a compile-time fact because the tile bookkeeping of the two layouts
+// Template parameters: which position terms exist, the element type, whether far key steps are looked for, the
+// layout (VARLEN: packed sequences) and the form of the position terms (STRIP: the caller's strips, not tables).  The layout is a compile-time fact because the tile bookkeeping of the two layouts
 // has nothing in common: with both compiled into one instance, the unused one still cost scalar registers (spilled
 // into vector lanes and reloaded in the step loops) and several hundred scalar instructions per tile.
-template <bool HAS_C2P, bool HAS_P2C, int DT, bool FARZ, bool VARLEN>
+template <bool HAS_C2P, bool HAS_P2C, int DT, bool FARZ, bool VARLEN, bool STRIP = false>
 __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelParams p, const int nblocks) {
+    static_assert(!(STRIP && FARZ), "the strip instances have no far steps");
     using E = Elem<DT>;
     using ET = typename E::T;
     using X2 = typename E::X2;
@@ -317,8 +324,8 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     auto k_of = [&](const Tile& t) {
         return static_cast<const uint16_t*>(p.k) + (VARLEN ? t.tok0 * p.ks_l : int64_t(t.b) * p.ks_b) + int64_t(t.head) * p.ks_h;
     };
-    auto pk_of = [&](const Tile& t) { return HAS_C2P ? static_cast<const uint16_t*>(p.pk) + int64_t(t.head) * p.pks_h : nullptr; };
-    auto pq_of = [&](const Tile& t) { return HAS_P2C ? static_cast<const uint16_t*>(p.pq) + int64_t(t.head) * p.pqs_h : nullptr; };
+    auto pk_of = [&](const Tile& t) { return HAS_C2P && !STRIP ? static_cast<const uint16_t*>(p.pk) + int64_t(t.head) * p.pks_h : nullptr; };
+    auto pq_of = [&](const Tile& t) { return HAS_P2C && !STRIP ? static_cast<const uint16_t*>(p.pq) + int64_t(t.head) * p.pqs_h : nullptr; };
 
     auto next_tile = [&](const Tile& t) {
         if constexpr (balanced) return take();
@@ -409,7 +416,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     {
         const int row = tid >> 3, ch = tid & 7;     // rows 0..63
         int dl[WIN / 64] = {0, 0, 0};
-        if (HAS_POS) {
+        if (HAS_POS && !STRIP) {
 #pragma unroll
             for (int n = 0; n < WIN / 64; ++n) dl[n] = delta_of(row0 - (BN - 1) + row + 64 * n);
             if (!score_role) {
@@ -425,19 +432,144 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         u32x4 wk[WIN / 64], wq[WIN / 64];
 #pragma unroll
         for (int n = 0; n < WIN / 64; ++n) {
-            if (HAS_C2P) wk[n] = *reinterpret_cast<const u32x4*>(PK + int64_t(dl[n]) * p.pks_r + ch * 8);
-            if (HAS_P2C) wq[n] = *reinterpret_cast<const u32x4*>(PQ + int64_t(dl[n]) * p.pqs_r + ch * 8);
+            if (HAS_C2P && !STRIP) wk[n] = *reinterpret_cast<const u32x4*>(PK + int64_t(dl[n]) * p.pks_r + ch * 8);
+            if (HAS_P2C && !STRIP) wq[n] = *reinterpret_cast<const u32x4*>(PQ + int64_t(dl[n]) * p.pqs_r + ch * 8);
         }
         *reinterpret_cast<u32x4*>(&sm.k[0][row * RS + ch * 8]) = k0;
         *reinterpret_cast<u32x4*>(&sm.k[1][row * RS + ch * 8]) = k1;
 #pragma unroll
         for (int n = 0; n < WIN / 64; ++n) {
-            if (HAS_C2P) *reinterpret_cast<u32x4*>(&sm.kr[(row + 64 * n) * RS + ch * 8]) = wk[n];
-            if (HAS_P2C) *reinterpret_cast<u32x4*>(&sm.qr[(row + 64 * n) * RS + ch * 8]) = wq[n];
+            if (HAS_C2P && !STRIP) *reinterpret_cast<u32x4*>(&sm.kr[(row + 64 * n) * RS + ch * 8]) = wk[n];
+            if (HAS_P2C && !STRIP) *reinterpret_cast<u32x4*>(&sm.qr[(row + 64 * n) * RS + ch * 8]) = wq[n];
         }
     }
 
-    if (!score_role) {
+    if constexpr (STRIP) {
+        if (!score_role) {
+            // ============================== position waves, strip instances =======================================
+            // The caller has the position terms as strips: c2p[i][delta] = Q_i.K_r[delta] per query row, p2c[j][delta] =
+            // K_j.Q_r[delta] per key row.  These waves only move them: for key step s they gather
+            //   ring[query i][key j mod 192] = c2p[i][delta(i - j)]     (128 queries x 64 keys), and
+            //   P'[key jl][x]               = p2c[j][delta(r_x)],  r_x = row0 - 64s + x - 63  (x = i - jl + 63, 128 per key)
+            // into the same LDS layouts the score waves read in the table instances, with the same barriers.  A lane is
+            // a key (c2p) or a window position x (p2c), so a load reads neighbouring columns of one strip row.  Rows
+            // past the end of the sequence read as zeros (buffer range check); the column comes from the delta table,
+            // whose values lie in [0, 2*span).
+            const int stid = tid - 256, srow = stid >> 3, sch = stid & 7;
+            const int c2s_bytes = int(p.c2s_l) * 2, p2s_bytes = int(p.p2s_l) * 2;
+            __amdgpu_buffer_rsrc_t c_rsrc, p_rsrc;
+            auto bind_strips = [&](const Tile& t) {
+                const uint16_t* cbase = HAS_C2P ? static_cast<const uint16_t*>(p.c2p) + (VARLEN ? t.tok0 * p.c2s_l : int64_t(t.b) * p.c2s_b) + int64_t(t.head) * p.c2s_h
+                                                : k_of(t);
+                const uint16_t* pbase = HAS_P2C ? static_cast<const uint16_t*>(p.p2c) + (VARLEN ? t.tok0 * p.p2s_l : int64_t(t.b) * p.p2s_b) + int64_t(t.head) * p.p2s_h
+                                                : k_of(t);
+                const bool any = t.vb >= 0 && t.len > 0;
+                c_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(cbase), 0, HAS_C2P && any ? (t.len - 1) * c2s_bytes + 4 * p.span : 0, RSRC_FLAGS);
+                p_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(pbase), 0, HAS_P2C && any ? (t.len - 1) * p2s_bytes + 4 * p.span : 0, RSRC_FLAGS);
+            };
+            uint16_t cv[32], pv[32];
+            // c2p of key step s of the tile at query row r0: this wave takes queries r0 + 32w + t, lane l is key 64s + l
+            auto gather_c = [&](int r0, int s) {
+                if (HAS_C2P) {
+                    // Column of (query q0 + t, lane l): delta(q0 + t - 64s - l).  Going from one query to the next every
+                    // lane takes over the column of its lower neighbour (a shift of the whole wave by one lane) and
+                    // lane 0 takes delta(q0 + t + 1 - 64s), which lane t of `ahead` has held since before the loop: two
+                    // reads of the delta table per step and wave instead of one per element.
+                    const int q0 = r0 + 32 * w;
+                    int d = delta_of(q0 - BN * s - l);
+                    const int ahead = delta_of(q0 + 1 + l - BN * s);
+#pragma unroll
+                    for (int t = 0; t < 32; ++t) {
+                        cv[t] = uint16_t(__builtin_amdgcn_raw_buffer_load_b16(c_rsrc, (q0 + t) * c2s_bytes + 2 * d, 0, 0));
+                        if (t < 31) d = __builtin_amdgcn_update_dpp(__builtin_amdgcn_readlane(ahead, t), d, 0x138 /* wave_shr:1 */, 0xf, 0xf, false);
+                    }
+                }
+            };
+            // ring row of tile row 4n + ws is 32 ws + n; the slots of step s start at (64 s) mod 192
+            auto write_c = [&](int phase) {
+                if (HAS_C2P) {
+#pragma unroll
+                    for (int t = 0; t < 32; ++t) sm.c[(32 * (t & 3) + 8 * w + (t >> 2)) * CRS + phase + l] = cv[t];
+                }
+            };
+            // p2c of key step s: this wave takes keys 64s + 16w + u; per key one load for x = 64 + l and one for
+            // x = l (lanes l >= 63 - jl) or x = 128 + l (the others) -- together the 128 positions the key is read at
+            auto gather_p = [&](int r0, int s) {
+                if (HAS_P2C) {
+                    int dx[3];
+#pragma unroll
+                    for (int c = 0; c < 3; ++c) dx[c] = 2 * delta_of(r0 - BN * s - (BN - 1) + 64 * c + l);
+#pragma unroll
+                    for (int u = 0; u < 16; ++u) {
+                        const int jl = 16 * w + u;
+                        const int rowoff = (BN * s + jl) * p2s_bytes;
+                        const int dsel = l + jl >= BN - 1 ? dx[0] : dx[2];
+                        pv[2 * u] = uint16_t(__builtin_amdgcn_raw_buffer_load_b16(p_rsrc, rowoff + dsel, 0, 0));
+                        pv[2 * u + 1] = uint16_t(__builtin_amdgcn_raw_buffer_load_b16(p_rsrc, rowoff + dx[1], 0, 0));
+                    }
+                }
+            };
+            auto write_p = [&]() {
+                if (HAS_P2C) {
+#pragma unroll
+                    for (int u = 0; u < 16; ++u) {
+                        const int jl = 16 * w + u;
+                        sm.p[jl * PS + (l + jl >= BN - 1 ? l : 2 * BN + l)] = pv[2 * u];
+                        sm.p[jl * PS + BN + l] = pv[2 * u + 1];
+                    }
+                }
+            };
+            auto next_phase = [](int ph) { return ph == 2 * BN ? 0 : ph + BN; };
+            bind_strips(cur);
+            gather_c(cur.row0, 0);
+            gather_p(cur.row0, 0);
+            phase_barrier();              // first stage of the first tile is in LDS
+            while (true) {
+                write_c(0);               // position terms of step 0 (gathered during the last step of the tile before)
+                write_p();
+                phase_barrier();          // the two opening barriers of the table instances
+                phase_barrier();
+                const Tile nxt = next_tile(cur);
+                int phase = BN;
+                for (int s = 0; s + 1 < nsteps; ++s) {
+                    phase_barrier();      // position terms of step s complete
+                    gather_c(row0, s + 1);
+                    gather_p(row0, s + 1);
+                    write_c(phase);       // (these ring slots were last read three steps ago)
+                    phase_barrier();      // the score waves are done with the scratch
+                    write_p();
+                    phase = next_phase(phase);
+                }
+                // Last key step: the next tile moves in -- its keys of steps 0 and 1 into both key buffers, its first
+                // position terms into registers (they go to LDS once the score waves have read this step's).
+                phase_barrier();
+                {
+                    const uint16_t* Kt = k_of(nxt);
+                    u32x4 st_k[4];
+#pragma unroll
+                    for (int n = 0; n < 4; ++n) {
+                        st_k[n] = u32x4{0, 0, 0, 0};
+                        if (nxt.vb >= 0) st_k[n] = *reinterpret_cast<const u32x4*>(Kt + int64_t(min(srow + 32 * n, nxt.len - 1)) * p.ks_l + sch * 8);
+                    }
+                    if (nxt.vb >= 0) {
+                        bind_strips(nxt);
+                        gather_c(nxt.row0, 0);
+                        gather_p(nxt.row0, 0);
+#pragma unroll
+                        for (int n = 0; n < 4; ++n)
+                            *reinterpret_cast<u32x4*>(&sm.k[n >> 1][(srow + 32 * (n & 1)) * RS + sch * 8]) = st_k[n];
+                    }
+                }
+                phase_barrier();
+                if (nxt.vb < 0) break;
+                cur = nxt;
+                bind(cur);
+            }
+            return;
+        }
+    }
+
+    if (!STRIP && !score_role) {
         // ================================================= position waves ==========================================
         const int stid = tid - 256;
         const int srow = stid >> 3, sch = stid & 7;          // this thread stages rows srow + 32n (chunk sch)
@@ -1149,11 +1281,15 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
 }  // namespace
 
 bool tdb_mfma_supported(const TdbKernelParams& p, int dtype) {
-    // bf16 or fp16, head_dim 64, position terms as fused tables (or none); strips go to the generic kernel.
-    // Buffer loads address rows with 32-bit byte offsets from the start of a (sequence, head).
-    if ((dtype != TDB_BF16 && dtype != TDB_F16) || p.D != 64 || p.c2p || p.p2c) return false;
+    // bf16 or fp16, head_dim 64, position terms as fused tables or as strips (or none); a call that mixes the two
+    // forms goes to the generic kernel.  Buffer loads address rows with 32-bit byte offsets from the start of a
+    // (sequence, head).
+    if ((dtype != TDB_BF16 && dtype != TDB_F16) || p.D != 64) return false;
+    if ((p.c2p || p.p2c) && (p.pk || p.pq)) return false;
     const int64_t lim = int64_t(1) << 31;
     const int64_t rows = p.L;
+    if (p.c2p && (rows * p.c2s_l * 2 + int64_t(4) * p.span >= lim || p.c2s_l < 0)) return false;
+    if (p.p2c && (rows * p.p2s_l * 2 + int64_t(4) * p.span >= lim || p.p2s_l < 0)) return false;
     if (rows * p.ks_l * 2 >= lim || rows * p.vs_l * 2 >= lim) return false;
     if (p.pk && int64_t(2) * p.span * p.pks_r * 2 >= lim) return false;
     if (p.pq && int64_t(2) * p.span * p.pqs_r * 2 >= lim) return false;
@@ -1166,7 +1302,7 @@ namespace {
 // ids are dealt over) and, per kernel instance, whether its dynamic-LDS limit has been raised on that device.
 constexpr int kMaxDevices = 64;
 constexpr int FAR_MIN_LEN = 1536;
-constexpr int kInstances = 32;
+constexpr int kInstances = 64;      // 32 for tables (layout, far, type, c2p, p2c), the strip instances above them
 std::mutex g_dev_mutex;
 int g_cus[kMaxDevices] = {0};
 bool g_attr_set[kMaxDevices][kInstances] = {{false}};
@@ -1202,14 +1338,16 @@ hipError_t tdb_launch_mfma(const TdbKernelParams& whole, int dtype, hipStream_t 
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;
     if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
-    const bool c2p = p.pk != nullptr, p2c = p.pq != nullptr;
+    const bool strip = p.c2p != nullptr || p.p2c != nullptr;
+    const bool c2p = strip ? p.c2p != nullptr : p.pk != nullptr, p2c = strip ? p.p2c != nullptr : p.pq != nullptr;
     // Far key steps only exist in sequences longer than the table's reach; the instance that looks for them carries
     // both step bodies and its near steps take 1.12x the time, a far step 0.65x.  At length 1024 a quarter of the steps
     // are far and the plain instance is 7 % faster; at 1536 the far instance wins by 2 %, at 4096 by 13 %.
-    const bool farz = (c2p || p2c) && p.L >= FAR_MIN_LEN;
+    const bool farz = !strip && (c2p || p2c) && p.L >= FAR_MIN_LEN;
     const int64_t round = int64_t(8) << (farz ? XG_LONG : XG_PLAIN);     // the id regrouping is a bijection on multiples of this
     const int nblocks = int((tiles + round - 1) / round * round);
-    const int instance = (p.varlen ? 16 : 0) + (farz ? 8 : 0) + (dtype == TDB_F16 ? 4 : 0) + (c2p ? 2 : 0) + (p2c ? 1 : 0);
+    const int instance = (p.varlen ? 16 : 0) + (farz ? 8 : 0) + (dtype == TDB_F16 ? 4 : 0) + (c2p ? 2 : 0) + (p2c ? 1 : 0) +
+                         (strip ? 32 : 0);
     const size_t smem = sizeof(Smem);
     const void* fn = nullptr;
 #define TDB_PICK(A, B, T)                                                                                        \
@@ -1217,9 +1355,16 @@ hipError_t tdb_launch_mfma(const TdbKernelParams& whole, int dtype, hipStream_t 
                           : reinterpret_cast<const void*>(&attn_mfma_kernel<A, B, T, true, false>))              \
               : (p.varlen ? reinterpret_cast<const void*>(&attn_mfma_kernel<A, B, T, false, true>)               \
                           : reinterpret_cast<const void*>(&attn_mfma_kernel<A, B, T, false, false>))
+#define TDB_PICK_STRIP(A, B, T)                                                                                  \
+    fn = p.varlen ? reinterpret_cast<const void*>(&attn_mfma_kernel<A, B, T, false, true, true>)                 \
+                  : reinterpret_cast<const void*>(&attn_mfma_kernel<A, B, T, false, false, true>)
 #define TDB_PICK_T(T)                                      \
     do {                                                   \
-        if (c2p && p2c) TDB_PICK(true, true, T);           \
+        if (strip) {                                       \
+            if (c2p && p2c) TDB_PICK_STRIP(true, true, T); \
+            else if (c2p) TDB_PICK_STRIP(true, false, T);  \
+            else TDB_PICK_STRIP(false, true, T);           \
+        } else if (c2p && p2c) TDB_PICK(true, true, T);    \
         else if (c2p) TDB_PICK(true, false, T);            \
         else if (p2c) TDB_PICK(false, true, T);            \
         else TDB_PICK(false, false, T);                    \
@@ -1227,6 +1372,7 @@ hipError_t tdb_launch_mfma(const TdbKernelParams& whole, int dtype, hipStream_t 
     if (dtype == TDB_F16) TDB_PICK_T(TDB_F16);
     else TDB_PICK_T(TDB_BF16);
 #undef TDB_PICK_T
+#undef TDB_PICK_STRIP
 #undef TDB_PICK
     int cus = 0;
     {
