@@ -56,6 +56,8 @@ RECORDED_TRAFFIC = {
     "varlen": "profiles/attn_mfma_kernel_varlen_64seq.md",
     "long": "profiles/attn_mfma_kernel_long_b4xL4096.md",
     "long_varlen": "profiles/attn_mfma_kernel_long_b4xL4096.md",
+    "strips_b32xL512": "profiles/attn_mfma_kernel_strips_b32xL512.md",
+    "strips_b8xL256": "profiles/attn_mfma_kernel_strips_b32xL512.md",
 }
 KERNEL_SOURCES = ("turbodeberta_amd/csrc/attn_mfma.hip", "turbodeberta_amd/csrc/tdb_internal.h")
 

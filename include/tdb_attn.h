@@ -52,7 +52,8 @@ extern "C" {
  *          with Q / K on the matrix cores; no [L, 2*span] strip ever exists in HBM.
  *  strip   c2p_strip / p2c_strip point at the strips the reference glue materialises
  *          (model.py:122-125, :146-148): Q.K_r^T and K.Q_r^T, [batch, heads, L, 2*span]
- *          (fixed) or [total, heads, 2*span] (varlen).  The kernel only gathers from them.
+ *          (fixed) or [total, heads, 2*span] (varlen).  The kernel only gathers from them
+ *          (on the matrix-core kernel when both terms are 16-bit strips and head_dim is 64).
  *
  * For score position (i, j) both terms use column delta(i - j) = delta_lut[i - j + lut_half],
  * the clamp(bucket(i - j) + span, 0, 2*span - 1) of Hugging Face's eager code
