@@ -81,6 +81,37 @@ def test_config2_fixed_b32_l512():
     assert torch.equal(outp, out[perm])
 
 
+def test_config2_strip_signature_b32_l512():
+    """The reference's own call at config 2: the glue's two strip matmuls (model.py:122-125, :146-148), then the
+    operator with `q_pos` / `k_pos`.  Oracle on a sample; against the table signature on the whole tensor (the two
+    differ by the bf16 rounding of the strips); packed strips == padded strips bit for bit on the valid rows."""
+    B, L = 32, 512
+    lengths = np.random.RandomState(0).randint(384, 513, size=B)
+    q, k, v, pk, pq = _projected(B, L)
+    lens = torch.from_numpy(lengths.astype(np.int32)).to(DEV)
+    c2p = torch.matmul(q, pk.transpose(-1, -2)[None])                    # [B, H, L, 2*span] bf16, 201 MB each
+    p2c = torch.matmul(k, pq.transpose(-1, -2)[None])
+    print("[case] config 2 strips", flush=True)
+    out = flash_attention_with_disentangled(q, k, v, c2p, p2c, False, SCALE, BUCKETS, MAX_REL, seqlens_k=lens)
+    torch.cuda.synchronize()
+    for b in sorted({int(lengths.argmin()), int(lengths.argmax())}):
+        n = int(lengths[b])
+        assert_close_bf16(out[b, :, :n], _oracle_rows(q, k, v, pk, pq, b, n), f"config 2 strips seq {b}", tol=1e-2)
+    pad = torch.arange(L, device=DEV)[None, :] >= lens[:, None]
+    assert torch.all(out.permute(0, 2, 1, 3)[pad] == 0)
+    print("[case] config 2 tables, for comparison", flush=True)
+    tab = flash_attention_with_disentangled(q, k, v, None, None, False, SCALE, BUCKETS, MAX_REL, pos_key_layer=pk,
+                                            pos_query_layer=pq, seqlens_k=lens)
+    assert (out.float() - tab.float()).abs().max().item() <= 1e-2
+    valid = ~pad
+    pack = lambda t: t.permute(0, 2, 1, 3)[valid].contiguous()            # [T, H, *]
+    cu = torch.from_numpy(np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)).to(DEV)
+    print("[case] config 2 strips, packed", flush=True)
+    outv = flash_attention_with_disentangled_varlen(pack(q), pack(k), pack(v), pack(c2p), pack(p2c), cu, cu, L, L,
+                                                    False, SCALE, BUCKETS, MAX_REL)
+    assert torch.equal(outv, pack(out))
+
+
 def test_config3_varlen_64_sequences():
     lengths = np.random.RandomState(0).randint(16, 513, size=64)
     T = int(lengths.sum())
