@@ -367,6 +367,59 @@ def test_fp16_varlen_matrix_core_equals_vector_alu():
         assert_close_bf16(outs[-1], ref, f"fp16 varlen generic={gen}", tol=2e-3)
 
 
+# ------------------------------------------------------------------ padded batches in the projection layout
+
+def _as_projection_output(t):
+    """The same values stored as [B, L, H, D] and viewed as [B, H, L, D]: what a projection followed by a head split
+    gives."""
+    return t.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,H,L,lengths", [
+    (5, 3, 400, (400, 1, 129, 256, 37)),        # whole tiles of padding (zeros from the up-front fill) and partial ones
+    (2, 12, 512, (512, 389)),
+    (3, 2, 128, (0, 128, 5)),                   # an empty sequence
+    (70, 1, 130, None),                         # more than 64 sequences: several launches
+    (2, 1, 2200, (2111, 1700)),                 # the instances with far key steps
+])
+def test_padded_projection_layout_equals_head_major_layout(B, H, L, lengths, dtype):
+    """A right-padded batch (a call with lengths: its tiles are dealt like those of packed sequences, its rows addressed
+    through the batch strides) gives the same bits whether its tensors are stored [B, L, H, D] or [B, H, L, D], and
+    matches the oracle; padded rows are zeros in both, whole tiles of them included."""
+    buckets, max_rel = 256, 512
+    if lengths is None:
+        lengths = tuple(int(x) for x in np.random.RandomState(B).randint(0, L + 1, size=B))
+    inp = make_inputs(31, B, H, L, 64, buckets, max_rel, dtype=dtype, lengths=lengths)
+    head_major = run_fixed(inp, buckets, max_rel)
+    proj = dict(inp)
+    for n in "qkv":
+        proj[n] = _as_projection_output(inp[n])
+        assert proj[n].stride(0) == L * proj[n].stride(2)
+    row_major = run_fixed(proj, buckets, max_rel)
+    assert torch.equal(row_major, head_major)
+    for b, n in enumerate(lengths):
+        assert torch.all(row_major[b, :, n:] == 0)
+    if L <= 512 and B <= 8:
+        ref = oracle_fixed(inp, buckets, max_rel, dtype=torch.float32)
+        assert_close_bf16(row_major, ref, "padded projection layout vs fp32 oracle", tol=1e-2 if dtype == torch.bfloat16 else 2e-3)
+
+
+def test_padded_projection_layout_with_strips():
+    B, H, L, buckets, max_rel = 4, 2, 300, 256, 512
+    lengths = (300, 40, 170, 129)
+    inp = make_inputs(32, B, H, L, 64, buckets, max_rel, dtype=torch.bfloat16, lengths=lengths)
+    c2p, p2c = _strips(inp)
+    head_major = _run_strips(inp, c2p, p2c, buckets, max_rel)
+    proj = dict(inp)
+    for n in "qkv":
+        proj[n] = _as_projection_output(inp[n])
+    row_major = _run_strips(proj, _as_projection_output(c2p), _as_projection_output(p2c), buckets, max_rel)
+    assert torch.equal(row_major, head_major)
+    for b, n in enumerate(lengths):
+        assert torch.all(row_major[b, :, n:] == 0)
+
+
 # ------------------------------------------------------------------ 16-bit strips (the reference's own operator signature)
 
 def _strips(inp, types=("c2p", "p2c")):

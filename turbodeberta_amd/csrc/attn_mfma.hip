@@ -153,6 +153,9 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     extern __shared__ __attribute__((aligned(16))) char smem_raw[];
     Smem& sm = *reinterpret_cast<Smem*>(smem_raw);
     constexpr bool HAS_POS = HAS_C2P || HAS_P2C;
+    // The packed instances also take right-padded batches of a fixed layout (lengths in p.seqlens, no cu_seqlens): the
+    // tiles are dealt like those of packed sequences, the rows are addressed through the batch strides.
+    const bool packed_rows = VARLEN && !p.seqlens;
 
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -213,7 +216,10 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     constexpr bool balanced = VARLEN;
     {
         int n = p.L, lo = 0;
-        if (VARLEN) {
+        if (VARLEN && p.seqlens) {
+            // right-padded sequences of a fixed layout, dealt like packed ones (the launcher sends such calls here)
+            n = l < p.B ? min(max(p.seqlens[min(l, p.B - 1)], 0), p.L) : 0;
+        } else if (VARLEN) {
             lo = p.cu_seqlens[min(l, p.B)];
             const int hi = p.cu_seqlens[min(l + 1, p.B)];
             n = hi - lo;
@@ -322,7 +328,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         return t;
     };
     auto k_of = [&](const Tile& t) {
-        return static_cast<const uint16_t*>(p.k) + (VARLEN ? t.tok0 * p.ks_l : int64_t(t.b) * p.ks_b) + int64_t(t.head) * p.ks_h;
+        return static_cast<const uint16_t*>(p.k) + (packed_rows ? t.tok0 * p.ks_l : int64_t(t.b) * p.ks_b) + int64_t(t.head) * p.ks_h;
     };
     auto pk_of = [&](const Tile& t) { return HAS_C2P && !STRIP ? static_cast<const uint16_t*>(p.pk) + int64_t(t.head) * p.pks_h : nullptr; };
     auto pq_of = [&](const Tile& t) { return HAS_P2C && !STRIP ? static_cast<const uint16_t*>(p.pq) + int64_t(t.head) * p.pqs_h : nullptr; };
@@ -341,6 +347,20 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         return delta_of(b) == delta_of(b + WIN - 2);
     };
 
+    if (VARLEN && p.seqlens) {
+        // The deal only lists tiles with valid query rows; tiles that hold padded rows alone get their zeros here,
+        // shared out over the workgroups (every thread fills its share of a tile's rows).
+        const int per_seq = (p.L + BM - 1) / BM;
+        for (int idx = blockIdx.x; idx < p.B * p.H * per_seq; idx += gridDim.x) {
+            const int bb = idx / (p.H * per_seq), rem = idx - bb * (p.H * per_seq);
+            const int hd = rem / per_seq, r0 = (rem - hd * per_seq) * BM;
+            if (r0 < lds_int(&sm.seq_n[bb])) continue;
+            uint16_t* Oz = static_cast<uint16_t*>(p.o) + int64_t(bb) * p.os_b + int64_t(hd) * p.os_h;
+            const int rows = min(BM, p.L - r0);
+            for (int i2 = tid; i2 < rows * (D / 8); i2 += NTHREADS)
+                *reinterpret_cast<u32x4*>(Oz + int64_t(r0 + (i2 >> 3)) * p.os_l + (i2 & 7) * 8) = u32x4{0, 0, 0, 0};
+        }
+    }
     Tile cur;
     if constexpr (balanced) cur = first_balanced();
     else cur = find_tile(blockIdx.x);
@@ -384,11 +404,11 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
         len = t.len;
         nsteps = (len + BN - 1) / BN;
         nfull = len / BN;                 // steps that need no key mask
-        rows_here = min(BM, (VARLEN ? len : p.L) - row0);   // rows of this tile that exist in memory
-        Q = static_cast<const uint16_t*>(p.q) + (VARLEN ? t.tok0 * p.qs_l : int64_t(t.b) * p.qs_b) + int64_t(t.head) * p.qs_h;
+        rows_here = min(BM, (packed_rows ? len : p.L) - row0);   // rows of this tile that exist in memory
+        Q = static_cast<const uint16_t*>(p.q) + (packed_rows ? t.tok0 * p.qs_l : int64_t(t.b) * p.qs_b) + int64_t(t.head) * p.qs_h;
         K = k_of(t);
-        V = static_cast<const uint16_t*>(p.v) + (VARLEN ? t.tok0 * p.vs_l : int64_t(t.b) * p.vs_b) + int64_t(t.head) * p.vs_h;
-        O = static_cast<uint16_t*>(p.o) + (VARLEN ? t.tok0 * p.os_l : int64_t(t.b) * p.os_b) + int64_t(t.head) * p.os_h;
+        V = static_cast<const uint16_t*>(p.v) + (packed_rows ? t.tok0 * p.vs_l : int64_t(t.b) * p.vs_b) + int64_t(t.head) * p.vs_h;
+        O = static_cast<uint16_t*>(p.o) + (packed_rows ? t.tok0 * p.os_l : int64_t(t.b) * p.os_b) + int64_t(t.head) * p.os_h;
         PK = pk_of(t);
         PQ = pq_of(t);
     };
@@ -397,7 +417,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
     // Q^T fragments of query block w: B operand of S^T = K.Q^T (score wave) and of C'^T = K_r'.Q^T (position wave)
     X8 qb[4];
     auto load_q = [&](X8 (&dst)[4], const Tile& t) {
-        const uint16_t* Qt = static_cast<const uint16_t*>(p.q) + (VARLEN ? t.tok0 * p.qs_l : int64_t(t.b) * p.qs_b) + int64_t(t.head) * p.qs_h;
+        const uint16_t* Qt = static_cast<const uint16_t*>(p.q) + (packed_rows ? t.tok0 * p.qs_l : int64_t(t.b) * p.qs_b) + int64_t(t.head) * p.qs_h;
         const int qrow = t.row0 + 4 * il + w;
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
@@ -459,9 +479,9 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
             const int c2s_bytes = int(p.c2s_l) * 2, p2s_bytes = int(p.p2s_l) * 2;
             __amdgpu_buffer_rsrc_t c_rsrc, p_rsrc;
             auto bind_strips = [&](const Tile& t) {
-                const uint16_t* cbase = HAS_C2P ? static_cast<const uint16_t*>(p.c2p) + (VARLEN ? t.tok0 * p.c2s_l : int64_t(t.b) * p.c2s_b) + int64_t(t.head) * p.c2s_h
+                const uint16_t* cbase = HAS_C2P ? static_cast<const uint16_t*>(p.c2p) + (packed_rows ? t.tok0 * p.c2s_l : int64_t(t.b) * p.c2s_b) + int64_t(t.head) * p.c2s_h
                                                 : k_of(t);
-                const uint16_t* pbase = HAS_P2C ? static_cast<const uint16_t*>(p.p2c) + (VARLEN ? t.tok0 * p.p2s_l : int64_t(t.b) * p.p2s_b) + int64_t(t.head) * p.p2s_h
+                const uint16_t* pbase = HAS_P2C ? static_cast<const uint16_t*>(p.p2c) + (packed_rows ? t.tok0 * p.p2s_l : int64_t(t.b) * p.p2s_b) + int64_t(t.head) * p.p2s_h
                                                 : k_of(t);
                 const bool any = t.vb >= 0 && t.len > 0;
                 c_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(cbase), 0, HAS_C2P && any ? (t.len - 1) * c2s_bytes + 4 * p.span : 0, RSRC_FLAGS);
@@ -1081,7 +1101,7 @@ __global__ __launch_bounds__(NTHREADS) void attn_mfma_kernel(const TdbKernelPara
             // keys of step 2 and values of step 0 of the next tile: its first half A stores them, and a first touch of
             // a new sequence takes longer than the opening of a tile lasts
             if (nxt.vb >= 0)
-                fetch_kv_from(k_of(nxt), static_cast<const uint16_t*>(p.v) + (VARLEN ? nxt.tok0 * p.vs_l : int64_t(nxt.b) * p.vs_b) + int64_t(nxt.head) * p.vs_h,
+                fetch_kv_from(k_of(nxt), static_cast<const uint16_t*>(p.v) + (packed_rows ? nxt.tok0 * p.vs_l : int64_t(nxt.b) * p.vs_b) + int64_t(nxt.head) * p.vs_h,
                               nxt.len, 2, 0);
         }
         if (s + 1 < nsteps) fetch_kv(s + 3, s + 1);   // for the next half A (nothing left to fetch in the last step)
@@ -1325,12 +1345,36 @@ hipError_t tdb_launch_mfma(const TdbKernelParams& whole, int dtype, hipStream_t 
         const int parts = (whole.B + 63) / 64, per = (whole.B + parts - 1) / parts;
         for (int first = 0; first < whole.B; first += per) {
             TdbKernelParams part = whole;
-            part.cu_seqlens = whole.cu_seqlens + first;
+            if (whole.cu_seqlens) {
+                part.cu_seqlens = whole.cu_seqlens + first;
+            } else {                      // a padded batch dealt like packed sequences (below): the part starts `first` sequences in
+                auto at = [first](const void* base, int64_t stride_b) { return base ? static_cast<const uint16_t*>(base) + first * stride_b : nullptr; };
+                part.seqlens = whole.seqlens + first;
+                part.q = at(whole.q, whole.qs_b);
+                part.k = at(whole.k, whole.ks_b);
+                part.v = at(whole.v, whole.vs_b);
+                part.o = const_cast<uint16_t*>(at(whole.o, whole.os_b));
+                part.c2p = at(whole.c2p, whole.c2s_b);
+                part.p2c = at(whole.p2c, whole.p2s_b);
+            }
             part.B = whole.B - first < per ? whole.B - first : per;
             const hipError_t e = tdb_launch_mfma(part, dtype, stream);
             if (e != hipSuccess) return e;
         }
         return hipSuccess;
+    }
+    // A fixed-layout call with valid lengths is a batch of sequences of different cost, and the strided walk of the
+    // fixed instances gives a workgroup the same (sequence, tile) in every head: the launch takes what its longest
+    // sequence takes, however short the others are.  Such a call goes to the packed instances, whose deal balances
+    // tiles of different cost (b32 x L512: lengths U[64,512] 0.092 -> 0.053 ms, U[384,512] 0.0934 -> 0.0915 ms); they
+    // address its rows through the batch strides and padded rows still come back as zeros.  Calls without lengths
+    // (every tile costs the same) keep the fixed instances.
+    if (!whole.varlen && whole.seqlens && int64_t(whole.B) * whole.L < (int64_t(1) << 31)) {
+        TdbKernelParams packed = whole;
+        packed.varlen = 1;
+        packed.cu_seqlens = nullptr;
+        packed.total = whole.B * whole.L;        // (sizes the upper bound of the tile count)
+        return tdb_launch_mfma(packed, dtype, stream);
     }
     const TdbKernelParams& p = whole;
     const int64_t tiles = int64_t(p.varlen ? p.total / BM + p.B : p.B * ((p.L + BM - 1) / BM)) * p.H;
