@@ -6,6 +6,8 @@ A "step" is one attention forward over one batch of synthetic DeBERTa-v3-base at
 
   fixed   batch 32 x seq 512, right-padded, valid lengths uniform in [384, 512]   (headline `value`)
   varlen  64 sequences with lengths uniform in [16, 512], packed with cu_seqlens  (reported beside it)
+  padded  batch 32 x seq 512 as in `fixed`, but with valid lengths uniform in [64, 512]: a padded batch as it reaches
+          the operator when nothing packs it   (`fixed_wide`, part of `all`)
   long    batch 4 x seq 4096, full mask, and its packed variant (8 sequences U[1024, 4096])   (`long`, `long_varlen`)
   strips  the reference's own call signature -- c2p / p2c strips [B, H, L, 2*span] computed by the caller -- on the
           matrix-core kernel: batch 8 x seq 256 and batch 32 x seq 512, bf16, priced against HBM (the strips are
@@ -132,10 +134,10 @@ def position_tables(w):
     return pk, pq
 
 
-def build_fixed(dev, B=32, L=512):
+def build_fixed(dev, B=32, L=512, shortest=384):
     from turbodeberta_amd.ops import flash_attention as fa
     w, g = make_weights(dev)
-    lengths = np.random.RandomState(0).randint(384, 513, size=B)
+    lengths = np.random.RandomState(0).randint(shortest, 513, size=B)
     hidden = torch.randn(B, L, HID, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
     lin = torch.nn.functional.linear
     heads = lambda x: x.view(B, L, H, D).permute(0, 2, 1, 3)       # projection-native storage, [B,H,L,D] view
@@ -451,6 +453,12 @@ def main():
         plan_v, lengths_v = build_varlen(dev)
         res_var = measure(plan_v, lengths_v, "varlen", "attn_mfma_kernel<c2p,p2c>")
     extra = {}
+    if args.workload == "all":
+        plan_w, lengths_w, _ = build_fixed(dev, shortest=64)
+        extra["fixed_wide"] = {"workload": "fixed b32xL512, valid lengths U[64,512] seed 0 (%d valid tokens), 12 heads x 64, c2p|p2c"
+                                           % int(lengths_w.sum()),
+                               **measure(plan_w, lengths_w, "fixed_wide", "attn_mfma_kernel<c2p,p2c>")}
+        del plan_w
     if args.workload in ("all", "long"):
         few = max(5, min(args.steps, 40))                      # a launch takes ~1 ms: fewer steps keep the run short
         plan_l, lengths_l = build_long(dev)
