@@ -298,7 +298,7 @@ def test_repeated_launches_are_bit_identical():
 
 def test_packed_tile_deal_at_other_grid_sizes():
     """The packed launch deals its tiles to the persistent workgroups inside the kernel.  Grids of 8, 24 and 40
-    workgroups (24 and 40 are not multiples of 16: teams of one) and the full device must all produce every tile:
+    workgroups and the full device must all produce every tile:
     the output is zero-filled first, so a tile that nobody took would stay zero, and each result must equal the
     full-grid one bit for bit (a tile's arithmetic does not depend on who computes it)."""
     from turbodeberta_amd import _lib
@@ -403,6 +403,29 @@ def test_padded_projection_layout_equals_head_major_layout(B, H, L, lengths, dty
     if L <= 512 and B <= 8:
         ref = oracle_fixed(inp, buckets, max_rel, dtype=torch.float32)
         assert_close_bf16(row_major, ref, "padded projection layout vs fp32 oracle", tol=1e-2 if dtype == torch.bfloat16 else 2e-3)
+
+
+def test_padded_batch_at_other_grid_sizes():
+    """A padded batch with whole tiles of padding at grids of 8, 40 and 248 workgroups: the deal and the up-front fill of
+    the padded tiles are both strided over the grid, and every grid must give the full-grid result bit for bit (the
+    output is allocated uninitialised, so a tile nobody filled would show)."""
+    from turbodeberta_amd import _lib
+    B, H, L, buckets, max_rel = 9, 5, 500, 256, 512
+    lengths = (500, 0, 3, 128, 129, 257, 384, 40, 499)
+    inp = make_inputs(33, B, H, L, 64, buckets, max_rel, dtype=torch.bfloat16, lengths=lengths)
+    try:
+        assert _lib.set_workgroup_limit(0) == 0
+        full = run_fixed(inp, buckets, max_rel)
+        assert_close_bf16(full, oracle_fixed(inp, buckets, max_rel, dtype=torch.float32), "padded batch, full grid", tol=1e-2)
+        for b, n in enumerate(lengths):
+            assert torch.all(full[b, :, n:] == 0)
+        for grid in (8, 40, 248):
+            assert _lib.set_workgroup_limit(grid) == grid
+            garbage = torch.full((64, 1024, 1024), 7.0, device=DEV)          # what the next allocations will reuse
+            del garbage
+            assert torch.equal(run_fixed(inp, buckets, max_rel), full), f"grid {grid}"
+    finally:
+        _lib.set_workgroup_limit(0)
 
 
 def test_padded_projection_layout_with_strips():
